@@ -1,0 +1,893 @@
+// Host side of the C ABI declared in include/bnn_hmc.h.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "bnn_device.h"
+#include "bnn_hmc.h"
+#include "bnn_kernels.h"
+#include "bnn_rng.h"
+
+namespace {
+
+using namespace bnn;
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                      \
+  do {                                                                                     \
+    hipError_t e_ = (expr);                                                                \
+    if (e_ != hipSuccess)                                                                  \
+      return fail(BNNHMC_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_),   \
+                  __FILE__, __LINE__);                                                     \
+  } while (0)
+
+// float constants from the double model constants, as the reference's lit<T>(double expr) does
+// (mcmc_step_ffma.h:289-300, 113-118; global_params.h:41-52)
+ModelConsts make_consts(const bnnhmc_model& m) {
+  const double pi = 3.14159265358979323846;
+  ModelConsts c;
+  c.scale_recp = (float)(1.0 / m.lik_scale);
+  c.df = (float)m.lik_df;
+  c.df_recp = m.lik_kind == BNNHMC_LIK_STUDENT_T ? (float)(1.0 / m.lik_df) : 0.0f;
+  if (m.lik_kind == BNNHMC_LIK_STUDENT_T) {
+    c.lik_norm = (float)(std::log(std::fabs(m.lik_scale)) + 0.5 * std::log(m.lik_df) +
+                         0.5 * std::log(pi) + std::lgamma(0.5 * m.lik_df) -
+                         std::lgamma(0.5 * (m.lik_df + 1.0)));
+  } else {
+    c.lik_norm = (float)(std::log(std::fabs(m.lik_scale)) + 0.5 * std::log(2.0 * pi));
+  }
+  c.l_scale = -0.5f * (c.df + 1.0f);
+  c.g_scale = (c.df + 1.0f) * c.scale_recp;
+  c.prior_recp = (float)(1.0 / m.prior_scale);
+  c.prior_norm = (float)(0.5 * std::log(2.0 * pi) + std::log(m.prior_scale));
+  c.prior_neg_recp2 = (float)(-1.0 / (m.prior_scale * m.prior_scale));
+  return c;
+}
+
+int check_model(const bnnhmc_model* m) {
+  if (!m) return fail(BNNHMC_ERR_INVALID, "model is null");
+  if (m->d0 != 22 || m->d1 != 40)
+    return fail(BNNHMC_ERR_INVALID, "unsupported layer sizes %d -> %d -> 1 (built: 22 -> 40 -> 1)",
+                m->d0, m->d1);
+  if (m->n <= 0) return fail(BNNHMC_ERR_INVALID, "n must be positive, got %d", m->n);
+  if (m->lik_kind != BNNHMC_LIK_STUDENT_T && m->lik_kind != BNNHMC_LIK_GAUSSIAN)
+    return fail(BNNHMC_ERR_INVALID, "unknown likelihood kind %d", m->lik_kind);
+  if (!(m->lik_scale > 0.0) || !(m->prior_scale > 0.0))
+    return fail(BNNHMC_ERR_INVALID, "scales must be positive");
+  if (m->lik_kind == BNNHMC_LIK_STUDENT_T && !(m->lik_df > 0.0))
+    return fail(BNNHMC_ERR_INVALID, "Student-t degrees of freedom must be positive");
+  return BNNHMC_OK;
+}
+
+struct DeviceInfo {
+  int n_devices = 0;
+  int cus = 0;
+  std::string arch;
+};
+
+int query_device(DeviceInfo& di) {
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return fail(BNNHMC_ERR_NO_DEVICE, "no HIP device visible (%s)",
+                e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+  }
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, 0));
+  di.n_devices = n;
+  di.cus = prop.multiProcessorCount;
+  di.arch = prop.gcnArchName;
+  if (di.arch.rfind("gfx950", 0) != 0)
+    return fail(BNNHMC_ERR_NO_DEVICE, "device 0 is %s; this library is built for gfx950 only",
+                di.arch.c_str());
+  return BNNHMC_OK;
+}
+
+// How a launch is laid over the GPU
+struct Plan {
+  const void* kernel = nullptr;
+  int threads = 0;
+  int G = 0;
+  int wgs_per_cu = 1;
+  int max_groups = 0;  // chain groups that can be co-resident
+  unsigned spin_limit = 1u << 22;
+  int transitions_per_launch = 8;
+};
+
+int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& di, Plan& p) {
+  bnnhmc_launch l;
+  bnnhmc_default_launch(&l);
+  if (lp) {
+    l.layer = lp->layer;
+    if (lp->cus_per_chain > 0) l.cus_per_chain = lp->cus_per_chain;
+    if (lp->wgs_per_cu > 0) l.wgs_per_cu = lp->wgs_per_cu;
+    if (lp->transitions_per_launch > 0) l.transitions_per_launch = lp->transitions_per_launch;
+    if (lp->spin_limit > 0) l.spin_limit = lp->spin_limit;
+  }
+  if (l.layer != BNNHMC_LAYER_MFMA && l.layer != BNNHMC_LAYER_FFMA)
+    return fail(BNNHMC_ERR_INVALID, "unknown layer variant %d", l.layer);
+  if (l.wgs_per_cu < 1 || l.wgs_per_cu > 2)
+    return fail(BNNHMC_ERR_INVALID, "wgs_per_cu must be 1 or 2, got %d", l.wgs_per_cu);
+  p.threads = (l.layer == BNNHMC_LAYER_MFMA && l.wgs_per_cu == 1) ? 512 : 256;
+  p.kernel = hmc_kernel_for(m.d0, m.d1, l.layer, m.lik_kind, p.threads);
+  if (!p.kernel) return fail(BNNHMC_ERR_INVALID, "no kernel for this configuration");
+  int per_cu = 0;
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, p.kernel, p.threads, 0));
+  if (per_cu < 1) return fail(BNNHMC_ERR_RESIDENCY, "kernel does not fit a compute unit");
+  p.wgs_per_cu = std::min(per_cu, l.wgs_per_cu);
+  p.G = l.cus_per_chain;
+  const int resident = p.wgs_per_cu * di.cus;
+  if (p.G > resident)
+    return fail(BNNHMC_ERR_RESIDENCY,
+                "%d workgroups per chain requested but only %d can be resident at once", p.G,
+                resident);
+  p.max_groups = resident / p.G;
+  p.spin_limit = l.spin_limit;
+  p.transitions_per_launch = l.transitions_per_launch;
+  return BNNHMC_OK;
+}
+
+size_t workspace_bytes_for(int P, int G, int groups) {
+  const size_t slot = (size_t)partial_slot_floats(P);
+  size_t bytes = (size_t)groups * 2 * G * slot * sizeof(float);          // partial records
+  bytes += (size_t)groups * BARRIER_STRIDE_WORDS * sizeof(unsigned);     // barrier words
+  bytes += 64 * sizeof(unsigned);                                        // status words
+  return bytes;
+}
+
+struct Workspace {
+  float* partials;
+  unsigned* barrier;
+  unsigned* status;
+};
+Workspace carve_workspace(void* base, int P, int G, int groups) {
+  Workspace w;
+  char* b = (char*)base;
+  w.partials = (float*)b;
+  b += (size_t)groups * 2 * G * partial_slot_floats(P) * sizeof(float);
+  w.barrier = (unsigned*)b;
+  b += (size_t)groups * BARRIER_STRIDE_WORDS * sizeof(unsigned);
+  w.status = (unsigned*)b;
+  return w;
+}
+
+void set_grid(KArgs& a, int groups, int G, int* workgroups) {
+  const int wgs = groups * G;
+  a.G = G;
+  a.n_groups = groups;
+  a.xcd_map = (wgs % 8 == 0) && ((wgs / 8) % G == 0) ? 1 : 0;
+  *workgroups = wgs;
+}
+
+// host restatement of the hidden activation (kernel_helpers.h:34-42) for the data generator
+inline float host_tanh(float x) {
+  const float e = exp2f(x * -2.88539008177792681472f);
+  const float sigm = 1.0f / (1.0f + e);
+  return std::fabs(x) < 0.0048176045529544353485f ? x : fmaf(sigm, 2.0f, -1.0f);
+}
+
+void generate_window_host(uint32_t seed, uint32_t window, int n, int d0, int d1, float teacher_scale,
+                          float noise_sigma, float* X, float* y, float* teacher) {
+  const Layout L = make_layout(d0, d1);
+  std::vector<float> th(L.P), h(d1);
+  for (int p = 0; p < L.P; ++p)
+    th[p] = teacher_scale * rng_normal(seed, window, STREAM_TEACHER, 0, (uint64_t)p);
+  if (teacher) memcpy(teacher, th.data(), sizeof(float) * L.P);
+  for (int i = 0; i < n; ++i) {
+    float* x = X + (size_t)i * d0;
+    for (int k = 0; k < d0; ++k) x[k] = rng_normal(seed, window, STREAM_X, 0, (uint64_t)i * d0 + k);
+    for (int c = 0; c < d1; ++c) h[c] = th[L.ob1 + c];
+    for (int k = 0; k < d0; ++k)
+      for (int c = 0; c < d1; ++c) h[c] = fmaf(th[(size_t)k * d1 + c], x[k], h[c]);
+    float yh = th[L.ob2];
+    for (int c = 0; c < d1; ++c) yh = fmaf(th[L.ow2 + c], host_tanh(h[c]), yh);
+    y[i] = fmaf(noise_sigma, rng_normal(seed, window, STREAM_NOISE, 0, (uint64_t)i), yh);
+  }
+}
+
+}  // namespace
+
+// =================================================================================================
+struct bnnhmc_sampler {
+  bnnhmc_model model;
+  bnnhmc_hmc hmc;
+  DeviceInfo dev;
+  Plan plan;
+  Layout L;
+  ModelConsts mc;
+  int n_windows = 0, cpw = 0, n_chains = 0;
+  int n_pad = 0;       // rows rounded up to 16
+  int st_stride = 0;   // floats per chain state record
+  int trace_len = 0;
+  bool data_set = false, inited = false;
+  std::vector<char> window_set;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  // device memory
+  float* X = nullptr;
+  float* y = nullptr;
+  float* st_w = nullptr;
+  float* st_g = nullptr;
+  float* st_eps = nullptr;
+  int* st_t = nullptr;
+  int* st_sel = nullptr;
+  int* st_nacc = nullptr;
+  float* ell0 = nullptr;
+  float* ell1 = nullptr;
+  float* samples = nullptr;
+  float* tr_la = nullptr;
+  int* tr_acc = nullptr;
+  float* tr_eps = nullptr;
+  void* workspace = nullptr;
+  size_t workspace_bytes = 0;
+  float* tmp = nullptr;       // evaluation scratch: w | grad | prior (3 * st_stride) ...
+  float* tmp_ell = nullptr;   // ... and n_pad rows
+  double* tmp_sums = nullptr; // [max_groups][2]
+  // timing
+  double kernel_ms = 0.0;
+  long launches = 0, grad_evals = 0;
+  int last_workgroups = 0;
+  int transitions_done = 0;
+
+  std::vector<void*> allocs;
+  template <typename T>
+  int alloc(T** p, size_t count) {
+    void* q = nullptr;
+    hipError_t e = hipMalloc(&q, std::max<size_t>(count, 1) * sizeof(T));
+    if (e != hipSuccess)
+      return fail(BNNHMC_ERR_HIP, "hipMalloc of %zu bytes failed: %s", count * sizeof(T),
+                  hipGetErrorString(e));
+    allocs.push_back(q);
+    *p = (T*)q;
+    return BNNHMC_OK;
+  }
+};
+
+namespace {
+
+KArgs base_args(const bnnhmc_sampler* s) {
+  KArgs a;
+  memset(&a, 0, sizeof(a));
+  a.n = s->model.n;
+  a.n_tiles = (s->model.n + 15) / 16;
+  a.mc = s->mc;
+  a.X = s->X;
+  a.y = s->y;
+  a.x_stride = (long)s->model.n * s->model.d0;
+  a.y_stride = s->n_pad;
+  a.x_vec_ok = (s->model.d0 % 2 == 0) ? 1 : 0;  // hipMalloc alignment, even row length
+  a.y_vec_ok = 1;                               // window stride is a multiple of 16 rows
+  a.chains_per_window = s->cpw;
+  a.fixed_window = -1;
+  a.L = s->hmc.leapfrog_steps;
+  a.spin_limit = s->plan.spin_limit;
+  Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.G, s->plan.max_groups);
+  a.partials = w.partials;
+  a.barrier = w.barrier;
+  a.status = w.status;
+  return a;
+}
+
+int launch_and_count(bnnhmc_sampler* s, KArgs& a, int groups) {
+  int wgs = 0;
+  set_grid(a, groups, s->plan.G, &wgs);
+  HIP_TRY(launch_fill_u32(a.barrier, (size_t)groups * BARRIER_STRIDE_WORDS, 0u, s->stream));
+  HIP_TRY(launch_hmc_kernel(s->plan.kernel, a, wgs, s->plan.threads, s->stream));
+  s->last_workgroups = wgs;
+  return BNNHMC_OK;
+}
+
+int check_status(bnnhmc_sampler* s) {
+  Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.G, s->plan.max_groups);
+  unsigned st[2] = {0, 0};
+  HIP_TRY(hipMemcpyAsync(st, w.status, sizeof(st), hipMemcpyDeviceToHost, s->stream));
+  HIP_TRY(hipStreamSynchronize(s->stream));
+  if (st[0] != 0) {
+    HIP_TRY(launch_fill_u32(w.status, 2, 0u, s->stream));
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    return fail(BNNHMC_ERR_TIMEOUT,
+                "a workgroup (%u) waited longer than the spin limit for its chain group; the launch "
+                "was abandoned",
+                st[1] ? st[1] - 1 : 0u);
+  }
+  return BNNHMC_OK;
+}
+
+// evaluate MODE_STEPS with L = 1, eps = 0 for `groups` parameter vectors starting at w_dev
+int eval_groups(bnnhmc_sampler* s, int window, const float* w_dev, long in_stride, int groups,
+                float* g_out, float* prior_out, long out_stride, float* ell_out, long ell_stride,
+                double* sums_out) {
+  KArgs a = base_args(s);
+  a.mode = MODE_STEPS;
+  a.L = 1;
+  a.eps_in = 0.0f;
+  a.fixed_window = window;
+  a.chain_base = 0;
+  a.w_in = w_dev;
+  a.in_stride = in_stride;
+  a.g_out = g_out;
+  a.prior_out = prior_out;
+  a.out_stride = out_stride;
+  a.ell_out = ell_out;
+  a.ell_stride = ell_stride;
+  a.sums_out = sums_out;
+  return launch_and_count(s, a, groups);
+}
+
+}  // namespace
+
+extern "C" {
+
+void bnnhmc_default_model(bnnhmc_model* m) {
+  if (!m) return;
+  m->d0 = 22;
+  m->d1 = 40;
+  m->n = 58368;
+  m->lik_kind = BNNHMC_LIK_STUDENT_T;
+  m->lik_scale = 100.0;
+  m->lik_df = 2.2;
+  m->prior_scale = 200.0;
+}
+
+void bnnhmc_default_hmc(bnnhmc_hmc* h) {
+  if (!h) return;
+  h->leapfrog_steps = 1000;
+  h->burn_in = 100;
+  h->n_samples = 800;
+  h->adapt_steps = 100;
+  h->eps0 = 0.01f;
+  h->target_rate = 0.2f;
+  h->decrement = 0.1f;
+  h->increment = 0.01f;
+  h->seed = 0;
+}
+
+void bnnhmc_default_launch(bnnhmc_launch* l) {
+  if (!l) return;
+  l->layer = BNNHMC_LAYER_MFMA;
+  l->cus_per_chain = 32;
+  l->wgs_per_cu = 1;
+  l->transitions_per_launch = 8;
+  l->spin_limit = 1u << 22;
+}
+
+int bnnhmc_num_params(int d0, int d1) { return make_layout(d0, d1).P; }
+
+const char* bnnhmc_last_error(void) { return g_last_error.c_str(); }
+
+int bnnhmc_device_info(int* n_devices, int* compute_units, char* arch, size_t arch_len) {
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    n = 0;
+  }
+  if (n_devices) *n_devices = n;
+  if (compute_units) *compute_units = 0;
+  if (arch && arch_len) arch[0] = 0;
+  if (n <= 0) return fail(BNNHMC_ERR_NO_DEVICE, "no HIP device visible");
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, 0));
+  if (compute_units) *compute_units = prop.multiProcessorCount;
+  if (arch && arch_len) {
+    strncpy(arch, prop.gcnArchName, arch_len - 1);
+    arch[arch_len - 1] = 0;
+  }
+  return BNNHMC_OK;
+}
+
+int bnnhmc_generate_window_host(uint32_t seed, uint32_t window, int n, int d0, int d1,
+                                float teacher_scale, float noise_sigma, float* x_out, float* y_out,
+                                float* teacher_out) {
+  if (n < 0 || d0 <= 0 || d1 <= 0 || !x_out || !y_out)
+    return fail(BNNHMC_ERR_INVALID, "bad arguments to bnnhmc_generate_window_host");
+  generate_window_host(seed, window, n, d0, d1, teacher_scale, noise_sigma, x_out, y_out,
+                       teacher_out);
+  return BNNHMC_OK;
+}
+
+// ---- host mirrors of the RNG, for callers that need the streams on the CPU ----
+uint32_t bnnhmc_rng_word(uint32_t seed, uint32_t id, uint32_t stream, uint32_t t, uint64_t index) {
+  return rng_word(seed, id, stream, t, index);
+}
+float bnnhmc_rng_normal(uint32_t seed, uint32_t id, uint32_t stream, uint32_t t, uint64_t index) {
+  return rng_normal(seed, id, stream, t, index);
+}
+float bnnhmc_rng_log_uniform(uint32_t seed, uint32_t chain_id, uint32_t t) {
+  return rng_log_uniform(seed, chain_id, t);
+}
+
+// =================================================================================================
+// operator level
+// =================================================================================================
+size_t bnnhmc_step_workspace_bytes(const bnnhmc_model* model, const bnnhmc_launch* launch) {
+  if (!model) return 0;
+  bnnhmc_launch l;
+  bnnhmc_default_launch(&l);
+  if (launch && launch->cus_per_chain > 0) l.cus_per_chain = launch->cus_per_chain;
+  return workspace_bytes_for(make_layout(model->d0, model->d1).P, l.cus_per_chain, 1);
+}
+
+int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, const float* x,
+                     const float* y, const float* weights_prev, float* weights_next,
+                     const float* mom_prev, float* mom_next, const float* grad_prev,
+                     float* grad_cur, float* grad_next, float* loss_values, void* workspace,
+                     size_t workspace_bytes, float eps, int lp_steps, void* stream) {
+  int rc = check_model(model);
+  if (rc) return rc;
+  if (!x || !y || !weights_prev || !weights_next || !mom_prev || !mom_next || !grad_prev ||
+      !grad_cur || !loss_values || !workspace)
+    return fail(BNNHMC_ERR_INVALID, "null device pointer passed to bnnhmc_mcmc_step");
+  if (lp_steps < 1) return fail(BNNHMC_ERR_INVALID, "lp_steps must be >= 1, got %d", lp_steps);
+  DeviceInfo di;
+  rc = query_device(di);
+  if (rc) return rc;
+  Plan plan;
+  rc = make_plan(*model, launch, di, plan);
+  if (rc) return rc;
+  const Layout L = make_layout(model->d0, model->d1);
+  if (workspace_bytes < workspace_bytes_for(L.P, plan.G, 1))
+    return fail(BNNHMC_ERR_INVALID, "workspace too small: %zu < %zu bytes", workspace_bytes,
+                workspace_bytes_for(L.P, plan.G, 1));
+  hipStream_t st = (hipStream_t)stream;
+  KArgs a;
+  memset(&a, 0, sizeof(a));
+  a.n = model->n;
+  a.n_tiles = (model->n + 15) / 16;
+  a.mc = make_consts(*model);
+  a.X = x;
+  a.y = y;
+  a.x_vec_ok = ((uintptr_t)x % 8 == 0 && model->d0 % 2 == 0) ? 1 : 0;
+  a.y_vec_ok = ((uintptr_t)y % 16 == 0) ? 1 : 0;
+  a.chains_per_window = 1;
+  a.fixed_window = 0;
+  a.mode = MODE_STEPS;
+  a.L = lp_steps;
+  a.eps_in = eps;
+  a.w_in = weights_prev;
+  a.m_in = mom_prev;
+  a.g_in = grad_prev;
+  a.w_out = weights_next;
+  a.m_out = mom_next;
+  a.g_out = grad_cur;
+  a.g_zero = grad_next;
+  a.ell_out = loss_values;
+  a.prior_out = loss_values + model->n;
+  a.spin_limit = plan.spin_limit;
+  Workspace w = carve_workspace(workspace, L.P, plan.G, 1);
+  a.partials = w.partials;
+  a.barrier = w.barrier;
+  a.status = w.status;
+  int wgs = 0;
+  set_grid(a, 1, plan.G, &wgs);
+  // barrier and status words start from zero on every call
+  HIP_TRY(launch_fill_u32(w.barrier, BARRIER_STRIDE_WORDS + 64, 0u, st));
+  HIP_TRY(launch_hmc_kernel(plan.kernel, a, wgs, plan.threads, st));
+  return BNNHMC_OK;
+}
+
+int bnnhmc_step_check(const bnnhmc_model* model, const bnnhmc_launch* launch, void* workspace,
+                      void* stream) {
+  if (!model || !workspace) return fail(BNNHMC_ERR_INVALID, "null argument to bnnhmc_step_check");
+  bnnhmc_launch l;
+  bnnhmc_default_launch(&l);
+  if (launch && launch->cus_per_chain > 0) l.cus_per_chain = launch->cus_per_chain;
+  Workspace w = carve_workspace(workspace, make_layout(model->d0, model->d1).P, l.cus_per_chain, 1);
+  unsigned st[2] = {0, 0};
+  HIP_TRY(hipMemcpyAsync(st, w.status, sizeof(st), hipMemcpyDeviceToHost, (hipStream_t)stream));
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  if (st[0] != 0)
+    return fail(BNNHMC_ERR_TIMEOUT, "workgroup %u waited longer than the spin limit; step abandoned",
+                st[1] ? st[1] - 1 : 0u);
+  return BNNHMC_OK;
+}
+
+int bnnhmc_sample_momentum(uint32_t seed, uint32_t chain_id, uint32_t transition, int n,
+                           float* prev_lp_mom, float* mom_next, void* stream) {
+  if (n < 0 || (n > 0 && !prev_lp_mom && !mom_next))
+    return fail(BNNHMC_ERR_INVALID, "bad arguments to bnnhmc_sample_momentum");
+  HIP_TRY(launch_sample_momentum(seed, chain_id, transition, n, prev_lp_mom, mom_next,
+                                 (hipStream_t)stream));
+  return BNNHMC_OK;
+}
+
+int bnnhmc_log_acpt(int n_loss, int n_mom, const float* prev_loss, const float* new_loss,
+                    const float* prev_mom, const float* new_mom, const float* grad_cur, float eps,
+                    float* log_acpt_out, float* host_out, void* stream) {
+  if (n_loss < 0 || n_mom < 0 || (n_loss > 0 && (!prev_loss || !new_loss)) ||
+      (n_mom > 0 && (!prev_mom || !new_mom || !grad_cur)))
+    return fail(BNNHMC_ERR_INVALID, "bad arguments to bnnhmc_log_acpt");
+  if (!log_acpt_out) return fail(BNNHMC_ERR_INVALID, "log_acpt_out (device) must not be null");
+  hipStream_t st = (hipStream_t)stream;
+  HIP_TRY(launch_log_acpt(n_loss, n_mom, prev_loss, new_loss, prev_mom, new_mom, grad_cur, eps,
+                          log_acpt_out, st));
+  if (host_out) {
+    HIP_TRY(hipMemcpyAsync(host_out, log_acpt_out, sizeof(float), hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipStreamSynchronize(st));
+  }
+  return BNNHMC_OK;
+}
+
+int bnnhmc_get_loss_values(const float* loss_values, int n, int n_params, float* loss1_host,
+                           float* loss2_host, void* stream) {
+  if (!loss_values || n < 0 || n_params < 0)
+    return fail(BNNHMC_ERR_INVALID, "bad arguments to bnnhmc_get_loss_values");
+  hipStream_t st = (hipStream_t)stream;
+  float* d = nullptr;
+  HIP_TRY(hipMalloc((void**)&d, 2 * sizeof(float)));
+  hipError_t e = launch_loss_sums(loss_values, n, n_params, d, st);
+  float h[2] = {0, 0};
+  if (e == hipSuccess) e = hipMemcpyAsync(h, d, sizeof(h), hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  (void)hipFree(d);
+  if (e != hipSuccess) return fail(BNNHMC_ERR_HIP, "loss sums failed: %s", hipGetErrorString(e));
+  if (loss1_host) *loss1_host = h[0];
+  if (loss2_host) *loss2_host = h[1];
+  return BNNHMC_OK;
+}
+
+// =================================================================================================
+// sampler level
+// =================================================================================================
+int bnnhmc_create(const bnnhmc_model* model, const bnnhmc_hmc* hmc, const bnnhmc_launch* launch,
+                  int n_windows, int chains_per_window, bnnhmc_sampler** out) {
+  if (!out) return fail(BNNHMC_ERR_INVALID, "out is null");
+  *out = nullptr;
+  int rc = check_model(model);
+  if (rc) return rc;
+  if (!hmc) return fail(BNNHMC_ERR_INVALID, "hmc is null");
+  if (hmc->leapfrog_steps < 1 || hmc->burn_in < 0 || hmc->n_samples < 0 || hmc->adapt_steps < 0)
+    return fail(BNNHMC_ERR_INVALID, "bad sampler constants");
+  if (n_windows < 1 || chains_per_window < 1)
+    return fail(BNNHMC_ERR_INVALID, "n_windows and chains_per_window must be >= 1");
+  DeviceInfo di;
+  rc = query_device(di);
+  if (rc) return rc;
+  bnnhmc_sampler* s = new (std::nothrow) bnnhmc_sampler();
+  if (!s) return fail(BNNHMC_ERR_INVALID, "out of host memory");
+  s->model = *model;
+  s->hmc = *hmc;
+  s->dev = di;
+  s->L = make_layout(model->d0, model->d1);
+  s->mc = make_consts(*model);
+  s->n_windows = n_windows;
+  s->cpw = chains_per_window;
+  s->n_chains = n_windows * chains_per_window;
+  s->n_pad = (model->n + 15) / 16 * 16;
+  s->st_stride = (s->L.P + 3) / 4 * 4;
+  s->trace_len = hmc->burn_in + hmc->n_samples;
+  s->window_set.assign(n_windows, 0);
+  rc = make_plan(*model, launch, di, s->plan);
+  if (rc) {
+    delete s;
+    return rc;
+  }
+  auto bail = [&](int code) {
+    bnnhmc_destroy(s);
+    return code;
+  };
+  hipError_t e = hipStreamCreate(&s->stream);
+  if (e == hipSuccess) e = hipEventCreate(&s->ev0);
+  if (e == hipSuccess) e = hipEventCreate(&s->ev1);
+  if (e != hipSuccess) {
+    fail(BNNHMC_ERR_HIP, "stream/event creation failed: %s", hipGetErrorString(e));
+    return bail(BNNHMC_ERR_HIP);
+  }
+  const size_t C = s->n_chains;
+  const int eval_groups_max = s->plan.max_groups;
+  s->workspace_bytes = workspace_bytes_for(s->L.P, s->plan.G, s->plan.max_groups);
+  char* ws = nullptr;
+  if ((rc = s->alloc(&s->X, (size_t)n_windows * model->n * model->d0)) ||
+      (rc = s->alloc(&s->y, (size_t)n_windows * s->n_pad)) ||
+      (rc = s->alloc(&s->st_w, C * s->st_stride)) || (rc = s->alloc(&s->st_g, C * s->st_stride)) ||
+      (rc = s->alloc(&s->st_eps, C)) || (rc = s->alloc(&s->st_t, C)) ||
+      (rc = s->alloc(&s->st_sel, C)) || (rc = s->alloc(&s->st_nacc, C)) ||
+      (rc = s->alloc(&s->ell0, C * s->n_pad)) || (rc = s->alloc(&s->ell1, C * s->n_pad)) ||
+      (rc = s->alloc(&s->samples, C * (size_t)hmc->n_samples * s->L.P)) ||
+      (rc = s->alloc(&s->tr_la, C * s->trace_len)) || (rc = s->alloc(&s->tr_acc, C * s->trace_len)) ||
+      (rc = s->alloc(&s->tr_eps, C * s->trace_len)) || (rc = s->alloc(&ws, s->workspace_bytes)) ||
+      (rc = s->alloc(&s->tmp, (size_t)3 * s->st_stride * eval_groups_max)) ||
+      (rc = s->alloc(&s->tmp_ell, (size_t)s->n_pad)) ||
+      (rc = s->alloc(&s->tmp_sums, (size_t)2 * eval_groups_max)))
+    return bail(rc);
+  s->workspace = ws;
+  e = hipMemsetAsync(s->y, 0, (size_t)n_windows * s->n_pad * sizeof(float), s->stream);
+  if (e == hipSuccess) e = hipMemsetAsync(ws, 0, s->workspace_bytes, s->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(s->stream);
+  if (e != hipSuccess) {
+    fail(BNNHMC_ERR_HIP, "clearing device memory failed: %s", hipGetErrorString(e));
+    return bail(BNNHMC_ERR_HIP);
+  }
+  *out = s;
+  return BNNHMC_OK;
+}
+
+int bnnhmc_destroy(bnnhmc_sampler* s) {
+  if (!s) return BNNHMC_OK;
+  if (s->stream) (void)hipStreamSynchronize(s->stream);
+  for (void* p : s->allocs) (void)hipFree(p);
+  if (s->ev0) (void)hipEventDestroy(s->ev0);
+  if (s->ev1) (void)hipEventDestroy(s->ev1);
+  if (s->stream) (void)hipStreamDestroy(s->stream);
+  delete s;
+  return BNNHMC_OK;
+}
+
+int bnnhmc_set_window_data(bnnhmc_sampler* s, int window, const float* x, const float* y) {
+  if (!s || !x || !y) return fail(BNNHMC_ERR_INVALID, "null argument to bnnhmc_set_window_data");
+  if (window < 0 || window >= s->n_windows)
+    return fail(BNNHMC_ERR_INVALID, "window %d out of range [0, %d)", window, s->n_windows);
+  const size_t nx = (size_t)s->model.n * s->model.d0;
+  HIP_TRY(hipMemcpyAsync(s->X + (size_t)window * nx, x, nx * sizeof(float), hipMemcpyHostToDevice,
+                         s->stream));
+  HIP_TRY(hipMemcpyAsync(s->y + (size_t)window * s->n_pad, y, (size_t)s->model.n * sizeof(float),
+                         hipMemcpyHostToDevice, s->stream));
+  HIP_TRY(hipStreamSynchronize(s->stream));
+  s->window_set[window] = 1;
+  return BNNHMC_OK;
+}
+
+int bnnhmc_generate_window(bnnhmc_sampler* s, int window, float teacher_scale, float noise_sigma,
+                           float* teacher_out) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  if (window < 0 || window >= s->n_windows)
+    return fail(BNNHMC_ERR_INVALID, "window %d out of range [0, %d)", window, s->n_windows);
+  std::vector<float> X((size_t)s->model.n * s->model.d0), y(s->model.n);
+  generate_window_host(s->hmc.seed, (uint32_t)window, s->model.n, s->model.d0, s->model.d1,
+                       teacher_scale, noise_sigma, X.data(), y.data(), teacher_out);
+  return bnnhmc_set_window_data(s, window, X.data(), y.data());
+}
+
+int bnnhmc_get_window_data(bnnhmc_sampler* s, int window, float* x_out, float* y_out) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  if (window < 0 || window >= s->n_windows)
+    return fail(BNNHMC_ERR_INVALID, "window %d out of range [0, %d)", window, s->n_windows);
+  const size_t nx = (size_t)s->model.n * s->model.d0;
+  if (x_out)
+    HIP_TRY(hipMemcpyAsync(x_out, s->X + (size_t)window * nx, nx * sizeof(float),
+                           hipMemcpyDeviceToHost, s->stream));
+  if (y_out)
+    HIP_TRY(hipMemcpyAsync(y_out, s->y + (size_t)window * s->n_pad,
+                           (size_t)s->model.n * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+  HIP_TRY(hipStreamSynchronize(s->stream));
+  return BNNHMC_OK;
+}
+
+int bnnhmc_init_chains(bnnhmc_sampler* s, const float* w0) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  for (int w = 0; w < s->n_windows; ++w)
+    if (!s->window_set[w])
+      return fail(BNNHMC_ERR_STATE, "window %d has no data (set_window_data / generate_window)", w);
+  const size_t C = s->n_chains;
+  std::vector<float> hw(C * s->st_stride, 0.0f);
+  if (w0)
+    for (size_t c = 0; c < C; ++c) memcpy(&hw[c * s->st_stride], w0, sizeof(float) * s->L.P);
+  HIP_TRY(hipMemcpyAsync(s->st_w, hw.data(), hw.size() * sizeof(float), hipMemcpyHostToDevice,
+                         s->stream));
+  HIP_TRY(launch_fill_f32(s->st_eps, C, s->hmc.eps0, s->stream));
+  HIP_TRY(launch_fill_u32((unsigned*)s->st_t, C, 0u, s->stream));
+  HIP_TRY(launch_fill_u32((unsigned*)s->st_sel, C, 0u, s->stream));
+  HIP_TRY(launch_fill_u32((unsigned*)s->st_nacc, C, 0u, s->stream));
+  // bootstrap (main.h:191-202): log-posterior rows and gradient at the initial state
+  for (int base = 0; base < s->n_chains; base += s->plan.max_groups) {
+    const int groups = std::min(s->plan.max_groups, s->n_chains - base);
+    KArgs a = base_args(s);
+    a.mode = MODE_STEPS;
+    a.L = 1;
+    a.eps_in = 0.0f;
+    a.chain_base = base;
+    a.w_in = s->st_w + (size_t)base * s->st_stride;
+    a.in_stride = s->st_stride;
+    a.g_out = s->st_g + (size_t)base * s->st_stride;
+    a.out_stride = s->st_stride;
+    a.ell_out = s->ell0 + (size_t)base * s->n_pad;
+    a.ell_stride = s->n_pad;
+    int rc = launch_and_count(s, a, groups);
+    if (rc) return rc;
+  }
+  int rc = check_status(s);
+  if (rc) return rc;
+  s->inited = true;
+  s->transitions_done = 0;
+  s->kernel_ms = 0.0;
+  s->launches = 0;
+  s->grad_evals = 0;
+  return BNNHMC_OK;
+}
+
+int bnnhmc_run(bnnhmc_sampler* s, int n_transitions) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  if (!s->inited) return fail(BNNHMC_ERR_STATE, "bnnhmc_init_chains has not been called");
+  if (n_transitions < 0) return fail(BNNHMC_ERR_INVALID, "n_transitions must be >= 0");
+  if (n_transitions == 0) return BNNHMC_OK;
+  long launches = 0;
+  HIP_TRY(hipEventRecord(s->ev0, s->stream));
+  for (int base = 0; base < s->n_chains; base += s->plan.max_groups) {
+    const int groups = std::min(s->plan.max_groups, s->n_chains - base);
+    for (int done = 0; done < n_transitions; done += s->plan.transitions_per_launch) {
+      KArgs a = base_args(s);
+      a.mode = MODE_TRANSITIONS;
+      a.n_trans = std::min(s->plan.transitions_per_launch, n_transitions - done);
+      a.chain_base = base;
+      a.st_w = s->st_w;
+      a.st_g = s->st_g;
+      a.st_stride = s->st_stride;
+      a.st_eps = s->st_eps;
+      a.st_t = s->st_t;
+      a.st_sel = s->st_sel;
+      a.st_nacc = s->st_nacc;
+      a.ell0 = s->ell0;
+      a.ell1 = s->ell1;
+      a.ell_stride = s->n_pad;
+      a.samples = s->samples;
+      a.n_samples = s->hmc.n_samples;
+      a.burn_in = s->hmc.burn_in;
+      a.adapt_steps = s->hmc.adapt_steps;
+      a.dec_adj = -s->hmc.decrement / (1.0f + s->hmc.decrement);
+      a.inc_adj = s->hmc.increment;
+      a.log_target = (float)std::log((double)s->hmc.target_rate);
+      a.tr_log_acpt = s->tr_la;
+      a.tr_accept = s->tr_acc;
+      a.tr_eps = s->tr_eps;
+      a.trace_len = s->trace_len;
+      a.seed = s->hmc.seed;
+      int rc = launch_and_count(s, a, groups);
+      if (rc) return rc;
+      ++launches;
+    }
+  }
+  HIP_TRY(hipEventRecord(s->ev1, s->stream));
+  int rc = check_status(s);
+  if (rc) return rc;
+  float ms = 0.0f;
+  HIP_TRY(hipEventElapsedTime(&ms, s->ev0, s->ev1));
+  s->kernel_ms += ms;
+  s->launches += launches;
+  s->grad_evals += (long)s->n_chains * n_transitions * s->hmc.leapfrog_steps;
+  s->transitions_done += n_transitions;
+  return BNNHMC_OK;
+}
+
+int bnnhmc_get_samples(bnnhmc_sampler* s, int chain, float* samples_out, int* n_stored) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  if (chain < 0 || chain >= s->n_chains)
+    return fail(BNNHMC_ERR_INVALID, "chain %d out of range [0, %d)", chain, s->n_chains);
+  const int stored =
+      std::max(0, std::min(s->hmc.n_samples, s->transitions_done - s->hmc.burn_in));
+  if (n_stored) *n_stored = stored;
+  if (samples_out && stored > 0) {
+    HIP_TRY(hipMemcpyAsync(samples_out, s->samples + (size_t)chain * s->hmc.n_samples * s->L.P,
+                           (size_t)stored * s->L.P * sizeof(float), hipMemcpyDeviceToHost,
+                           s->stream));
+    HIP_TRY(hipStreamSynchronize(s->stream));
+  }
+  return BNNHMC_OK;
+}
+
+int bnnhmc_get_chain_state(bnnhmc_sampler* s, int chain, float* w, float* grad, float* eps,
+                           int* transitions_done, int* n_accepted) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  if (chain < 0 || chain >= s->n_chains)
+    return fail(BNNHMC_ERR_INVALID, "chain %d out of range [0, %d)", chain, s->n_chains);
+  const size_t o = (size_t)chain * s->st_stride;
+  if (w) HIP_TRY(hipMemcpyAsync(w, s->st_w + o, s->L.P * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+  if (grad)
+    HIP_TRY(hipMemcpyAsync(grad, s->st_g + o, s->L.P * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+  if (eps) HIP_TRY(hipMemcpyAsync(eps, s->st_eps + chain, sizeof(float), hipMemcpyDeviceToHost, s->stream));
+  if (transitions_done)
+    HIP_TRY(hipMemcpyAsync(transitions_done, s->st_t + chain, sizeof(int), hipMemcpyDeviceToHost, s->stream));
+  if (n_accepted)
+    HIP_TRY(hipMemcpyAsync(n_accepted, s->st_nacc + chain, sizeof(int), hipMemcpyDeviceToHost, s->stream));
+  HIP_TRY(hipStreamSynchronize(s->stream));
+  return BNNHMC_OK;
+}
+
+int bnnhmc_get_traces(bnnhmc_sampler* s, int chain, float* log_acpt, int* accepted, float* eps) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  if (chain < 0 || chain >= s->n_chains)
+    return fail(BNNHMC_ERR_INVALID, "chain %d out of range [0, %d)", chain, s->n_chains);
+  const int len = std::min(s->transitions_done, s->trace_len);
+  const size_t o = (size_t)chain * s->trace_len;
+  if (len > 0) {
+    if (log_acpt)
+      HIP_TRY(hipMemcpyAsync(log_acpt, s->tr_la + o, len * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+    if (accepted)
+      HIP_TRY(hipMemcpyAsync(accepted, s->tr_acc + o, len * sizeof(int), hipMemcpyDeviceToHost, s->stream));
+    if (eps)
+      HIP_TRY(hipMemcpyAsync(eps, s->tr_eps + o, len * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+    HIP_TRY(hipStreamSynchronize(s->stream));
+  }
+  return BNNHMC_OK;
+}
+
+int bnnhmc_eval(bnnhmc_sampler* s, int window, const float* w, float* ell, float* prior,
+                float* grad) {
+  if (!s || !w) return fail(BNNHMC_ERR_INVALID, "null argument to bnnhmc_eval");
+  if (window < 0 || window >= s->n_windows)
+    return fail(BNNHMC_ERR_INVALID, "window %d out of range [0, %d)", window, s->n_windows);
+  if (!s->window_set[window]) return fail(BNNHMC_ERR_STATE, "window %d has no data", window);
+  float* dw = s->tmp;
+  float* dg = s->tmp + s->st_stride;
+  float* dp = s->tmp + 2 * s->st_stride;
+  HIP_TRY(hipMemcpyAsync(dw, w, s->L.P * sizeof(float), hipMemcpyHostToDevice, s->stream));
+  int rc = eval_groups(s, window, dw, 0, 1, dg, dp, 0, s->tmp_ell, 0, nullptr);
+  if (rc) return rc;
+  rc = check_status(s);
+  if (rc) return rc;
+  if (ell)
+    HIP_TRY(hipMemcpyAsync(ell, s->tmp_ell, (size_t)s->model.n * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+  if (prior)
+    HIP_TRY(hipMemcpyAsync(prior, dp, s->L.P * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+  if (grad)
+    HIP_TRY(hipMemcpyAsync(grad, dg, s->L.P * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+  HIP_TRY(hipStreamSynchronize(s->stream));
+  return BNNHMC_OK;
+}
+
+int bnnhmc_final_loss(bnnhmc_sampler* s, int chain, double* loss1, double* loss2, double* full) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  if (chain < 0 || chain >= s->n_chains)
+    return fail(BNNHMC_ERR_INVALID, "chain %d out of range [0, %d)", chain, s->n_chains);
+  const int stored =
+      std::max(0, std::min(s->hmc.n_samples, s->transitions_done - s->hmc.burn_in));
+  if (stored == 0) return fail(BNNHMC_ERR_STATE, "chain %d has no kept samples yet", chain);
+  const int window = chain / s->cpw;
+  const float* base = s->samples + (size_t)chain * s->hmc.n_samples * s->L.P;
+  std::vector<double> sums((size_t)2 * s->plan.max_groups);
+  double l1 = 0, l2 = 0, fl = 0;
+  int step = 0;
+  // the samples are evaluated max_groups at a time, one chain group per sample
+  for (int b = 0; b < stored; b += s->plan.max_groups) {
+    const int groups = std::min(s->plan.max_groups, stored - b);
+    int rc = eval_groups(s, window, base + (size_t)b * s->L.P, s->L.P, groups, nullptr, nullptr, 0,
+                         nullptr, 0, s->tmp_sums);
+    if (rc) return rc;
+    rc = check_status(s);
+    if (rc) return rc;
+    HIP_TRY(hipMemcpy(sums.data(), s->tmp_sums, (size_t)2 * groups * sizeof(double),
+                      hipMemcpyDeviceToHost));
+    for (int i = 0; i < groups; ++i, ++step) {
+      // running means as main.h:106-111; the reference's per-sample sums are FP32
+      const double s1 = (double)(float)sums[2 * i], s2 = (double)(float)sums[2 * i + 1];
+      const double ds = (double)step;
+      l1 = (l1 * ds + s1) / (ds + 1);
+      l2 = (l2 * ds + s2) / (ds + 1);
+      fl = (fl * ds + (s1 + s2)) / (ds + 1);
+    }
+  }
+  if (loss1) *loss1 = l1;
+  if (loss2) *loss2 = l2;
+  if (full) *full = fl;
+  return BNNHMC_OK;
+}
+
+int bnnhmc_get_timing(bnnhmc_sampler* s, double* kernel_ms, long* launches, long* grad_evals,
+                      int* workgroups) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  if (kernel_ms) *kernel_ms = s->kernel_ms;
+  if (launches) *launches = s->launches;
+  if (grad_evals) *grad_evals = s->grad_evals;
+  if (workgroups) *workgroups = s->last_workgroups;
+  return BNNHMC_OK;
+}
+
+}  // extern "C"

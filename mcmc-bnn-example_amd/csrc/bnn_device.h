@@ -1,0 +1,117 @@
+// Structures shared by the host side of the library and its kernels.
+#pragma once
+
+#include <stdint.h>
+
+namespace bnn {
+
+// parameter layout, include/mcmc/mcmc_step_ffma.h:35-44
+struct Layout {
+  int d0, d1, oW1, ob1, ow2, ob2, P;
+};
+inline Layout make_layout(int d0, int d1) {
+  Layout L;
+  L.d0 = d0;
+  L.d1 = d1;
+  L.oW1 = 0;
+  L.ob1 = d0 * d1;
+  L.ow2 = L.ob1 + d1;
+  L.ob2 = L.ow2 + d1;
+  L.P = L.ob2 + 1;
+  return L;
+}
+
+// float constants of the likelihood and the prior, derived on the host exactly as the reference
+// derives them from its double constexprs (mcmc_step_ffma.h:289-300, 113-118)
+struct ModelConsts {
+  float scale_recp;  // 1 / lik_scale
+  float df;
+  float df_recp;
+  float lik_norm;  // Student-t or Gaussian normalisation
+  float l_scale;   // -0.5 (df + 1)
+  float g_scale;   // (df + 1) / scale
+  float prior_recp;
+  float prior_norm;
+  float prior_neg_recp2;
+};
+
+enum KernelMode : int {
+  MODE_STEPS = 0,       // L leapfrog steps from given (w, m, g): the step operator / evaluation
+  MODE_TRANSITIONS = 1  // whole HMC transitions with RNG, accept, adaptation and sample store
+};
+
+// Number of floats of one workgroup's partial-result record: P gradient partials padded to a
+// multiple of 4, then 4 words of which the first two hold a double (sum of per-row log-likelihood
+// terms).
+inline int partial_slot_floats(int P) { return ((P + 3) / 4) * 4 + 4; }
+
+constexpr int BARRIER_STRIDE_WORDS = 32;  // one 128-byte line per chain group
+
+struct KArgs {
+  // ---- model / data ----
+  int n;        // rows per window
+  int n_tiles;  // ceil(n / 16)
+  ModelConsts mc;
+  const float* X;   // [window][n][d0]
+  const float* y;   // [window][y_stride]
+  long x_stride;    // floats between windows
+  long y_stride;
+  int x_vec_ok;     // X rows may be read with 8-byte loads
+  int y_vec_ok;     // y may be read with 16-byte loads
+  // ---- decomposition ----
+  int G;            // workgroups per chain group
+  int n_groups;     // chain groups in this launch
+  int chain_base;   // global chain index of group 0
+  int chains_per_window;
+  int fixed_window; // >= 0: every group reads this window
+  int xcd_map;      // 1: blockIdx is spread round-robin over 8 XCDs, keep a group inside one XCD
+  // ---- what to do ----
+  int mode;
+  int L;            // leapfrog steps per trajectory
+  int n_trans;      // MODE_TRANSITIONS: transitions in this launch
+  // ---- MODE_STEPS io (per group strides in floats; null inputs read as zero) ----
+  const float* w_in;
+  const float* m_in;
+  const float* g_in;
+  long in_stride;
+  float* w_out;
+  float* m_out;
+  float* g_out;
+  float* g_zero;      // zero-filled (the reference's grad_next)
+  long out_stride;
+  float* ell_out;     // per-row log-lik, [group][ell_stride]
+  long ell_stride;
+  float* prior_out;   // per-parameter log-prior, [group][out_stride]
+  double* sums_out;   // [group][2]: sum of ell, sum of log-prior
+  float eps_in;
+  // ---- MODE_TRANSITIONS state, indexed by global chain ----
+  float* st_w;        // [chain][PS]
+  float* st_g;        // [chain][PS]
+  long st_stride;
+  float* st_eps;      // [chain]
+  int* st_t;          // [chain] transitions done
+  int* st_sel;        // [chain] which ell buffer holds the current state's rows
+  int* st_nacc;       // [chain]
+  float* ell0;        // [chain][ell_stride]
+  float* ell1;
+  float* samples;     // [chain][n_samples][P]
+  int n_samples;
+  int burn_in;
+  int adapt_steps;
+  float dec_adj;      // -decrement / (1 + decrement)
+  float inc_adj;
+  float log_target;   // log(target_rate)
+  float* tr_log_acpt; // [chain][trace_len]
+  int* tr_accept;
+  float* tr_eps;
+  int trace_len;
+  uint32_t seed;
+  // ---- cross-workgroup exchange ----
+  float* partials;     // [group][2][G][slot]
+  unsigned* barrier;   // [group][BARRIER_STRIDE_WORDS]
+  unsigned* status;    // [0] abort flag, [1] timed-out workgroup + 1
+  unsigned spin_limit;
+  unsigned* debug_xcc; // optional [workgroup] XCC id
+};
+
+}  // namespace bnn

@@ -1,0 +1,906 @@
+// Fused HMC trajectory kernel for gfx950 (MI355X).
+//
+// One persistent launch integrates whole trajectories (and, in MODE_TRANSITIONS, whole HMC
+// transitions) for a batch of independent chains.  A chain's rows are shared by G workgroups
+// ("chain group"); every workgroup of the group redundantly integrates all P parameters, so only
+// the gradient crosses workgroups, once per leapfrog step, through a deterministic two-stage
+// reduction: (1) wavefront partials -> LDS slots -> fixed-order sum per workgroup, (2) per-workgroup
+// partials in global scratch -> group barrier -> fixed-order sum in every workgroup.
+//
+// What it replaces in the reference: leapfrog_step_kernel (include/mcmc/mcmc_step_ffma.h:154-379),
+// the persistent mcmc_step_kernel with its grid barrier (include/mcmc/mcmc_step_tc.h:597-677),
+// the momentum lambda, log_acpt_prec, the accept/restore copies, the step-size update and the
+// sample store of main_loop (include/mcmc/main.h:204-287).
+#include <hip/hip_runtime.h>
+
+#include "bnn_device.h"
+#include "bnn_kernels.h"
+#include "bnn_rng.h"
+
+namespace bnn {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+// ------------------------------------------------------------------------------------------------
+// small device helpers
+// ------------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+// sum over the 16 lanes of a DPP row; every lane of the row receives the same bits (each step adds
+// a value to its mirror image, and a + b == b + a)
+__device__ __forceinline__ float row16_allreduce(float v) {
+  v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_move<0x141>(v);  // row_half_mirror
+  v += dpp_move<0x140>(v);  // row_mirror
+  return v;
+}
+// sum over the 8 lanes of a half row
+__device__ __forceinline__ float row8_allreduce(float v) {
+  v += dpp_move<0xB1>(v);
+  v += dpp_move<0x4E>(v);
+  v += dpp_move<0x141>(v);
+  return v;
+}
+
+__device__ __forceinline__ double shfl_xor_d(double v, int mask) {
+  const uint64_t b = double_to_bits(v);
+  const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)b, mask);
+  const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(b >> 32), mask);
+  return bits_to_double(((uint64_t)hi << 32) | lo);
+}
+
+// activation of the hidden layer, include/mcmc/kernel_helpers.h:34-42:
+// tanh(x) = 2 sigmoid(2x) - 1 with e^(-2x) = 2^(x * -2/ln 2); identity below the cutoff
+__device__ __forceinline__ float tanh_fwd(float x) {
+  const float e = __builtin_amdgcn_exp2f(x * -2.88539008177792681472f);
+  const float sigm = __builtin_amdgcn_rcpf(1.0f + e);
+  const float r = __builtin_fmaf(sigm, 2.0f, -1.0f);
+  return __builtin_fabsf(x) < 0.0048176045529544353485f ? x : r;
+}
+
+// per-row log-likelihood gradient (and value) given the residual, mcmc_step_ffma.h:293-301
+template <int LIK>
+__device__ __forceinline__ float lik_grad(const ModelConsts& mc, float resid, float& diff_out) {
+  const float diff = resid * mc.scale_recp;
+  diff_out = diff;
+  if (LIK == 0) {
+    return diff * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(diff, diff, mc.df));
+  } else {
+    return diff * mc.scale_recp;
+  }
+}
+template <int LIK>
+__device__ __forceinline__ float lik_value(const ModelConsts& mc, float diff) {
+  if (LIK == 0) {
+    return mc.l_scale * log1pf(diff * diff * mc.df_recp) - mc.lik_norm;
+  } else {
+    return -0.5f * (diff * diff) - mc.lik_norm;
+  }
+}
+
+// prior terms, mcmc_step_ffma.h:113-118
+__device__ __forceinline__ float prior_logp(const ModelConsts& mc, float w) {
+  const float lp = w * mc.prior_recp;
+  return -(lp * lp) * 0.5f - mc.prior_norm;
+}
+__device__ __forceinline__ float prior_grad(const ModelConsts& mc, float w) {
+  return w * mc.prior_neg_recp2;
+}
+
+__device__ __forceinline__ float ld_agent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Per-wave working set handed to a layer for one leapfrog step
+// ------------------------------------------------------------------------------------------------
+struct StepCtx {
+  const float* X;        // this window's rows
+  const float* y;
+  int n;
+  int tile_begin, tile_end;  // 16-row tiles of this wave
+  bool x_vec_ok, y_vec_ok;
+  const float* ell_prev;  // last step only: rows of the current state (null = zeros)
+  float* ell_new;         // last step only: where to store this state's rows (null = skip)
+};
+
+// ================================================================================================
+// MFMA layer: both contractions on v_mfma_f32_16x16x4_f32.
+//
+// Lane l = 16 q + n (q = 0..3, n = 0..15).  A 16-row tile is processed as
+//   GEMM1  A = X_aug tile  [16 rows x K]   lane (n, q) holds row n, k = KS q + s      (s < KS)
+//          B = W1_aug      [K x 16 c]      lane (n, q) holds k = KS q + s, c = 16 t + n
+//          C = pre-act     [16 rows x 16 c] lane (n, q) holds rows 4 q + j, c = 16 t + n
+//   GEMM2  A = delta^T     [16 c x 4 rows]  = C layout of GEMM1 reused as is (k-step j <-> rows
+//                                             4 q + j): no shuffle between the two GEMMs
+//          B = X_aug tile  [4 rows x 16 f]  lane (n, q) holds row 4 q + j, features 2 n + u
+//          C = dW1_aug^T   [16 c x 16 f]    lane (n, q) holds c = 16 t + 4 q + j', f = 2 n + u
+// X_aug appends a constant-one feature (index D0) so that b1 rides in GEMM1 and db1 falls out of
+// GEMM2; the contraction index of GEMM1 and the feature index of GEMM2 are permuted so that every
+// lane reads contiguous floats of a row.
+// ================================================================================================
+template <int D0, int D1>
+struct MfmaLayer {
+  static_assert(D0 % 2 == 0, "feature pairs are read as float2");
+  static constexpr int KS = (D0 + 1 + 3) / 4;  // k-steps of GEMM1 (one more feature: the bias)
+  static_assert(KS % 2 == 0, "k-steps are read in pairs");
+  static constexpr int KP = KS / 2;
+  static constexpr int NT = (D1 + 15) / 16;  // hidden tiles
+  static_assert(D0 + 1 <= 32, "one feature-pair tile");
+  static constexpr int oB1 = D0 * D1, oW2 = oB1 + D1, oB2 = oW2 + D1, P = oB2 + 1;
+  static constexpr int P_AL = (P + 3) / 4 * 4;
+
+  float w1b[KS][NT];
+  float w2v[NT];
+  float b2;
+  f4 dacc[NT][2];
+  float dw2acc[NT];
+  float db2acc;
+  double dl;
+
+  struct TileIn {
+    f2 xa[KP];
+    f2 xb[4];
+    f4 yv;
+  };
+
+  __device__ __forceinline__ void load_weights(const float* s_w) {
+    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int c = 16 * t + n;
+      const bool cv = c < D1;
+      const int cc = cv ? c : 0;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int k = KS * q + s;
+        float v = 0.0f;
+        if (k < D0) v = s_w[k * D1 + cc];
+        else if (k == D0) v = s_w[oB1 + cc];
+        w1b[s][t] = cv ? v : 0.0f;
+      }
+      w2v[t] = cv ? s_w[oW2 + cc] : 0.0f;
+    }
+    b2 = s_w[oB2];
+  }
+
+  __device__ __forceinline__ void zero_acc() {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      dacc[t][0] = f4{0.f, 0.f, 0.f, 0.f};
+      dacc[t][1] = f4{0.f, 0.f, 0.f, 0.f};
+      dw2acc[t] = 0.0f;
+    }
+    db2acc = 0.0f;
+    dl = 0.0;
+  }
+
+  __device__ __forceinline__ void load_tile_fast(TileIn& ti, const StepCtx& cx, int row0, int n,
+                                                 int q) const {
+    const float* ra = cx.X + (size_t)(row0 + n) * D0;
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int k0 = KS * q + 2 * i;
+      const int kc = k0 < D0 ? k0 : D0 - 2;
+      f2 v = *reinterpret_cast<const f2*>(ra + kc);
+      if (k0 >= D0) v = f2{k0 == D0 ? 1.0f : 0.0f, 0.0f};
+      ti.xa[i] = v;
+    }
+    const int f0 = 2 * n;
+    const int fc = f0 < D0 ? f0 : D0 - 2;
+    const float* rb = cx.X + (size_t)(row0 + 4 * q) * D0 + fc;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f2 v = *reinterpret_cast<const f2*>(rb + j * D0);
+      if (f0 >= D0) v = f2{f0 == D0 ? 1.0f : 0.0f, 0.0f};
+      ti.xb[j] = v;
+    }
+    ti.yv = *reinterpret_cast<const f4*>(cx.y + row0 + 4 * q);
+  }
+
+  // any alignment, rows past the end read as the last row (their gradient is masked to zero)
+  __device__ __forceinline__ void load_tile_safe(TileIn& ti, const StepCtx& cx, int row0, int n,
+                                                 int q) const {
+    const int last = cx.n - 1;
+    const int rowa = min(row0 + n, last);
+    const float* ra = cx.X + (size_t)rowa * D0;
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int k0 = KS * q + 2 * i;
+      const int kc = k0 < D0 ? k0 : D0 - 2;
+      f2 v = f2{ra[kc], ra[kc + 1]};
+      if (k0 >= D0) v = f2{k0 == D0 ? 1.0f : 0.0f, 0.0f};
+      ti.xa[i] = v;
+    }
+    const int f0 = 2 * n;
+    const int fc = f0 < D0 ? f0 : D0 - 2;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int rowb = min(row0 + 4 * q + j, last);
+      const float* rb = cx.X + (size_t)rowb * D0 + fc;
+      f2 v = f2{rb[0], rb[1]};
+      if (f0 >= D0) v = f2{f0 == D0 ? 1.0f : 0.0f, 0.0f};
+      ti.xb[j] = v;
+      ti.yv[j] = cx.y[rowb];
+    }
+  }
+
+  __device__ __forceinline__ void load_tile(TileIn& ti, const StepCtx& cx, int tile, int n,
+                                            int q) const {
+    const int row0 = tile * 16;
+    if (cx.x_vec_ok && cx.y_vec_ok && row0 + 16 <= cx.n) load_tile_fast(ti, cx, row0, n, q);
+    else load_tile_safe(ti, cx, row0, n, q);
+  }
+
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void compute_tile(const TileIn& ti, const StepCtx& cx,
+                                               const ModelConsts& mc, int row0, int n, int q) {
+    // ---- GEMM1: pre-activations (bias included through the constant-one feature) ----
+    f4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(ti.xa[i][0], w1b[2 * i][t], acc[t], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] =
+            __builtin_amdgcn_mfma_f32_16x16x4f32(ti.xa[i][1], w1b[2 * i + 1][t], acc[t], 0, 0, 0);
+    }
+    // ---- activation, layer-2 dot ----
+    float yh[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[t][j] = tanh_fwd(acc[t][j]);
+        yh[j] = __builtin_fmaf(w2v[t], acc[t][j], yh[j]);
+      }
+    }
+    // ---- per-row loss gradient ----
+    float g[4];
+    float gsum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float yhat = row16_allreduce(yh[j]);
+      float diff;
+      float gj = lik_grad<LIK>(mc, ti.yv[j] - yhat - b2, diff);
+      const bool valid = row0 + 4 * q + j < cx.n;
+      gj = valid ? gj : 0.0f;  // mcmc_step_ffma.h:301
+      g[j] = gj;
+      gsum += gj;
+      if (LAST) {
+        if (n == 0 && valid) {
+          const int row = row0 + 4 * q + j;
+          const float lv = lik_value<LIK>(mc, diff);
+          const float prev = cx.ell_prev ? cx.ell_prev[row] : 0.0f;
+          if (cx.ell_new) cx.ell_new[row] = lv;
+          dl += (double)(lv - prev);
+        }
+      }
+    }
+    db2acc += gsum;
+    // ---- layer-2 weight gradient, delta = (1 - h^2) w2 g ----
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float h = acc[t][j];
+        dw2acc[t] = __builtin_fmaf(g[j], h, dw2acc[t]);
+        acc[t][j] = __builtin_fmaf(-h, h, 1.0f) * (w2v[t] * g[j]);
+      }
+    }
+    // ---- GEMM2: dW1_aug^T += delta^T X_aug ----
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        dacc[t][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(acc[t][j], ti.xb[j][0], dacc[t][0], 0, 0, 0);
+        dacc[t][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(acc[t][j], ti.xb[j][1], dacc[t][1], 0, 0, 0);
+      }
+    }
+  }
+
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void run_tiles(const StepCtx& cx, const ModelConsts& mc) {
+    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    if (cx.tile_begin >= cx.tile_end) return;
+    TileIn cur, nxt;
+    load_tile(cur, cx, cx.tile_begin, n, q);
+    for (int tile = cx.tile_begin; tile < cx.tile_end; ++tile) {
+      const int tn = tile + 1 < cx.tile_end ? tile + 1 : tile;
+      load_tile(nxt, cx, tn, n, q);  // prefetch
+      compute_tile<LIK, LAST>(cur, cx, mc, tile * 16, n, q);
+      cur = nxt;
+    }
+  }
+
+  // this wave's partial sums -> its LDS slot, indexed by canonical parameter number
+  __device__ __forceinline__ void write_partials(float* slot) {
+    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int f = 2 * n + u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int c = 16 * t + 4 * q + j;
+          if (c < D1) {
+            if (f < D0) slot[f * D1 + c] = dacc[t][u][j];
+            else if (f == D0) slot[oB1 + c] = dacc[t][u][j];
+          }
+        }
+      }
+      // dw2: sum the four row groups q in a fixed order
+      float v = dw2acc[t];
+      v += __shfl_xor(v, 16);
+      v += __shfl_xor(v, 32);
+      const int c = 16 * t + n;
+      if (q == 0 && c < D1) slot[oW2 + c] = v;
+    }
+    float b = db2acc;
+    b += __shfl_xor(b, 16);
+    b += __shfl_xor(b, 32);
+    double d = dl;  // held by lanes n == 0
+    d += shfl_xor_d(d, 16);
+    d += shfl_xor_d(d, 32);
+    if (lane == 0) {
+      slot[oB2] = b;
+      const uint64_t bits = double_to_bits(d);
+      slot[P_AL] = __builtin_bit_cast(float, (uint32_t)bits);
+      slot[P_AL + 1] = __builtin_bit_cast(float, (uint32_t)(bits >> 32));
+    }
+  }
+};
+
+// ================================================================================================
+// FFMA layer: both contractions on the vector ALU (v_fma_f32).
+//
+// Lane l = 8 rg + cc (rg = 0..7 row of an 8-row tile pair, cc = 0..7).  Lane (rg, cc) owns hidden
+// units c = cc + 8 i (i < HU) for the rows r0 + rg of each 8-row sub-tile: its W1 columns and its
+// dW1 accumulators stay in registers for the whole step, the row's features are read once and
+// broadcast by the memory system to the 8 lanes that share the row.
+// ================================================================================================
+template <int D0, int D1>
+struct FfmaLayer {
+  static_assert(D1 % 8 == 0, "hidden units are dealt to 8 lanes");
+  static_assert(D0 % 2 == 0, "feature pairs are read as float2");
+  static constexpr int HU = D1 / 8;
+  static constexpr int oB1 = D0 * D1, oW2 = oB1 + D1, oB2 = oW2 + D1, P = oB2 + 1;
+  static constexpr int P_AL = (P + 3) / 4 * 4;
+
+  float w1[D0][HU];
+  float b1[HU];
+  float w2[HU];
+  float b2;
+  float dw1[D0][HU];
+  float db1[HU];
+  float dw2[HU];
+  float db2acc;
+  double dl;
+
+  struct RowIn {
+    float x[D0];
+    float yv;
+  };
+
+  __device__ __forceinline__ void load_weights(const float* s_w) {
+    const int lane = threadIdx.x & 63, cc = lane & 7;
+#pragma unroll
+    for (int i = 0; i < HU; ++i) {
+      const int c = cc + 8 * i;
+#pragma unroll
+      for (int k = 0; k < D0; ++k) w1[k][i] = s_w[k * D1 + c];
+      b1[i] = s_w[oB1 + c];
+      w2[i] = s_w[oW2 + c];
+    }
+    b2 = s_w[oB2];
+  }
+
+  __device__ __forceinline__ void zero_acc() {
+#pragma unroll
+    for (int i = 0; i < HU; ++i) {
+#pragma unroll
+      for (int k = 0; k < D0; ++k) dw1[k][i] = 0.0f;
+      db1[i] = 0.0f;
+      dw2[i] = 0.0f;
+    }
+    db2acc = 0.0f;
+    dl = 0.0;
+  }
+
+  __device__ __forceinline__ void load_row(RowIn& ri, const StepCtx& cx, int row) const {
+    const int r = min(row, cx.n - 1);
+    const float* rp = cx.X + (size_t)r * D0;
+    if (cx.x_vec_ok) {
+#pragma unroll
+      for (int k = 0; k < D0; k += 2) {
+        const f2 v = *reinterpret_cast<const f2*>(rp + k);
+        ri.x[k] = v[0];
+        ri.x[k + 1] = v[1];
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < D0; ++k) ri.x[k] = rp[k];
+    }
+    ri.yv = cx.y[r];
+  }
+
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void compute_row(const RowIn& ri, const StepCtx& cx,
+                                              const ModelConsts& mc, int row, int cc) {
+    float h[HU];
+    // layer 1: FMA chain over k ascending from the bias (mcmc_step_ffma.h:225-255)
+#pragma unroll
+    for (int i = 0; i < HU; ++i) h[i] = b1[i];
+#pragma unroll
+    for (int k = 0; k < D0; ++k) {
+#pragma unroll
+      for (int i = 0; i < HU; ++i) h[i] = __builtin_fmaf(w1[k][i], ri.x[k], h[i]);
+    }
+    float yh = 0.0f;
+#pragma unroll
+    for (int i = 0; i < HU; ++i) {
+      h[i] = tanh_fwd(h[i]);
+      yh = __builtin_fmaf(w2[i], h[i], yh);
+    }
+    const float yhat = row8_allreduce(yh);
+    float diff;
+    float g = lik_grad<LIK>(mc, ri.yv - yhat - b2, diff);
+    const bool valid = row < cx.n;
+    g = valid ? g : 0.0f;
+    if (LAST) {
+      if (cc == 0 && valid) {
+        const float lv = lik_value<LIK>(mc, diff);
+        const float prev = cx.ell_prev ? cx.ell_prev[row] : 0.0f;
+        if (cx.ell_new) cx.ell_new[row] = lv;
+        dl += (double)(lv - prev);
+      }
+    }
+    db2acc += g;
+    float delta[HU];
+#pragma unroll
+    for (int i = 0; i < HU; ++i) {
+      dw2[i] = __builtin_fmaf(g, h[i], dw2[i]);
+      delta[i] = __builtin_fmaf(-h[i], h[i], 1.0f) * (w2[i] * g);
+      db1[i] += delta[i];
+    }
+#pragma unroll
+    for (int k = 0; k < D0; ++k) {
+#pragma unroll
+      for (int i = 0; i < HU; ++i) dw1[k][i] = __builtin_fmaf(ri.x[k], delta[i], dw1[k][i]);
+    }
+  }
+
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void run_tiles(const StepCtx& cx, const ModelConsts& mc) {
+    const int lane = threadIdx.x & 63, cc = lane & 7, rg = lane >> 3;
+    const int row_begin = cx.tile_begin * 16, row_end = min(cx.tile_end * 16, (cx.n + 7) / 8 * 8);
+    if (row_begin >= row_end) return;
+    RowIn cur, nxt;
+    load_row(cur, cx, row_begin + rg);
+    for (int r0 = row_begin; r0 < row_end; r0 += 8) {
+      const int rn = r0 + 8 < row_end ? r0 + 8 : r0;
+      load_row(nxt, cx, rn + rg);  // prefetch
+      compute_row<LIK, LAST>(cur, cx, mc, r0 + rg, cc);
+      cur = nxt;
+    }
+  }
+
+  // sum over the 8 row lanes rg (lane bits 3, 4, 5) in a fixed order
+  __device__ __forceinline__ float reduce_rg(float v) const {
+    v += __shfl_xor(v, 8);
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+  }
+
+  __device__ __forceinline__ void write_partials(float* slot) {
+    const int lane = threadIdx.x & 63, cc = lane & 7, rg = lane >> 3;
+#pragma unroll
+    for (int i = 0; i < HU; ++i) {
+      const int c = cc + 8 * i;
+#pragma unroll
+      for (int k = 0; k < D0; ++k) {
+        const float v = reduce_rg(dw1[k][i]);
+        if (rg == 0) slot[k * D1 + c] = v;
+      }
+      const float vb = reduce_rg(db1[i]);
+      const float vw = reduce_rg(dw2[i]);
+      if (rg == 0) {
+        slot[oB1 + c] = vb;
+        slot[oW2 + c] = vw;
+      }
+    }
+    const float b = reduce_rg(db2acc);  // every cc lane of a row holds the same g
+    double d = dl;                      // held by lanes cc == 0
+    d += shfl_xor_d(d, 8);
+    d += shfl_xor_d(d, 16);
+    d += shfl_xor_d(d, 32);
+    if (lane == 0) {
+      slot[oB2] = b;
+      const uint64_t bits = double_to_bits(d);
+      slot[P_AL] = __builtin_bit_cast(float, (uint32_t)bits);
+      slot[P_AL + 1] = __builtin_bit_cast(float, (uint32_t)(bits >> 32));
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------------------------
+// group barrier: all G workgroups of a chain group have published their partials of this step.
+// Bounded: after spin_limit polls, or when another workgroup has given up, the wait ends and the
+// launch is abandoned (status[0] set), so every wave always exits.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ bool group_barrier(unsigned* counter, unsigned target, unsigned* status,
+                                              unsigned spin_limit, int* s_flag) {
+  __syncthreads();  // this workgroup's partials are stored (and waited for)
+  if (threadIdx.x == 0) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned polls = 0;
+    int ok = 1;
+    while ((int)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
+      __builtin_amdgcn_s_sleep(2);
+      if ((++polls & 63u) == 0u) {
+        if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
+          ok = 0;
+          break;
+        }
+        if (polls >= spin_limit) {
+          __hip_atomic_store(status + 1, (unsigned)blockIdx.x + 1u, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          ok = 0;
+          break;
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    *s_flag = ok;
+  }
+  __syncthreads();
+  return *s_flag != 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// the kernel
+// ------------------------------------------------------------------------------------------------
+template <class Layer, int LIK, int T>
+__global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
+  constexpr int W = T / 64;
+  constexpr int P = Layer::P;
+  constexpr int P_AL = Layer::P_AL;
+  constexpr int SLOT = P_AL + 4;
+  constexpr int PPT = (P + T - 1) / T;
+
+  __shared__ float s_w[P_AL];
+  __shared__ float s_slots[W][SLOT];
+  __shared__ double s_red[W];
+  __shared__ int s_flag;
+
+  // ---- which chain group, which rank inside it ----
+  int lin = blockIdx.x;
+  if (a.xcd_map) {
+    const int per_xcd = gridDim.x >> 3;
+    lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  }
+  const int group = lin / a.G, rank = lin - group * a.G;
+  if (a.debug_xcc && threadIdx.x == 0) {
+    // XCC_ID hardware register (id 20), bits 3:0
+    a.debug_xcc[blockIdx.x] = __builtin_amdgcn_s_getreg((3 << 11) | 20);
+  }
+  if (group >= a.n_groups) return;
+  const int chain = a.chain_base + group;
+  const int window = a.fixed_window >= 0 ? a.fixed_window : chain / a.chains_per_window;
+  const int tid = threadIdx.x, wave = tid >> 6;
+
+  StepCtx cx;
+  cx.X = a.X + (size_t)window * a.x_stride;
+  cx.y = a.y + (size_t)window * a.y_stride;
+  cx.n = a.n;
+  cx.x_vec_ok = a.x_vec_ok != 0;
+  cx.y_vec_ok = a.y_vec_ok != 0;
+  {
+    const int gw = rank * W + wave, GW = a.G * W;
+    cx.tile_begin = (int)((long)a.n_tiles * gw / GW);
+    cx.tile_end = (int)((long)a.n_tiles * (gw + 1) / GW);
+  }
+  cx.ell_prev = nullptr;
+  cx.ell_new = nullptr;
+
+  const ModelConsts mc = a.mc;
+  float* part_base = a.partials + (size_t)group * 2 * a.G * SLOT;
+  unsigned* counter = a.barrier + (size_t)group * BARRIER_STRIDE_WORDS;
+  unsigned bar_target = 0;
+  int buf = 0;
+
+  // ---- parameters owned by this thread: p = tid + i T ----
+  float w[PPT], m[PPT], g[PPT], wc[PPT], gc[PPT], m0[PPT];
+  float eps;
+  int t0 = 0, sel = 0, nacc = 0;
+  const bool trans = a.mode == MODE_TRANSITIONS;
+#pragma unroll
+  for (int i = 0; i < PPT; ++i) {
+    const int p = tid + i * T;
+    w[i] = m[i] = g[i] = wc[i] = gc[i] = m0[i] = 0.0f;
+    if (p < P) {
+      if (trans) {
+        wc[i] = a.st_w[(size_t)chain * a.st_stride + p];
+        gc[i] = a.st_g[(size_t)chain * a.st_stride + p];
+      } else {
+        const size_t o = (size_t)group * a.in_stride + p;
+        w[i] = a.w_in ? a.w_in[o] : 0.0f;
+        m[i] = a.m_in ? a.m_in[o] : 0.0f;
+        g[i] = a.g_in ? a.g_in[o] : 0.0f;
+      }
+    }
+  }
+  if (trans) {
+    eps = a.st_eps[chain];
+    t0 = a.st_t[chain];
+    sel = a.st_sel[chain];
+    nacc = a.st_nacc[chain];
+  } else {
+    eps = a.eps_in;
+  }
+
+  Layer layer;
+  bool ok = true;
+  const int n_outer = trans ? a.n_trans : 1;
+  double dl_total = 0.0;
+
+  for (int it = 0; it < n_outer && ok; ++it) {
+    const uint32_t t = (uint32_t)(t0 + it);
+    float* ell_cur = nullptr;
+    float* ell_prop = nullptr;
+    if (trans) {
+      // momentum resampling (main.h:207-216); the start state is the last accepted one
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        const int p = tid + i * T;
+        if (p < P) {
+          m0[i] = rng_normal(a.seed, (uint32_t)chain, STREAM_MOMENTUM, t, (uint64_t)p);
+          m[i] = m0[i];
+          w[i] = wc[i];
+          g[i] = gc[i];
+        }
+      }
+      ell_cur = (sel ? a.ell1 : a.ell0) + (size_t)chain * a.ell_stride;
+      ell_prop = (sel ? a.ell0 : a.ell1) + (size_t)chain * a.ell_stride;
+    } else {
+      ell_prop = a.ell_out ? a.ell_out + (size_t)group * a.ell_stride : nullptr;
+    }
+
+    for (int s = 0; s < a.L && ok; ++s) {
+      // ---- leapfrog update (mcmc_step_ffma.h:106-112): half kick on the first step ----
+      const float ek = s == 0 ? eps * 0.5f : eps;
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        const int p = tid + i * T;
+        if (p < P) {
+          m[i] = __builtin_fmaf(ek, g[i], m[i]);
+          w[i] = __builtin_fmaf(eps, m[i], w[i]);
+          s_w[p] = w[i];
+        }
+      }
+      __syncthreads();
+      layer.load_weights(s_w);
+      layer.zero_acc();
+      const bool last = s == a.L - 1;
+      if (last) {
+        cx.ell_prev = ell_cur;
+        cx.ell_new = ell_prop;
+        layer.template run_tiles<LIK, true>(cx, mc);
+      } else {
+        layer.template run_tiles<LIK, false>(cx, mc);
+      }
+      layer.write_partials(s_slots[wave]);
+      __syncthreads();
+      // ---- stage 1: fixed-order sum over this workgroup's waves -> global partial record ----
+      float* my_part = part_base + ((size_t)buf * a.G + rank) * SLOT;
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        const int p = tid + i * T;
+        if (p < P) {
+          float v = s_slots[0][p];
+#pragma unroll
+          for (int wv = 1; wv < W; ++wv) v += s_slots[wv][p];
+          st_agent(my_part + p, v);
+        }
+      }
+      if (last && tid == 0) {
+        double d = 0.0;
+#pragma unroll
+        for (int wv = 0; wv < W; ++wv) {
+          const uint64_t bits = ((uint64_t)__builtin_bit_cast(uint32_t, s_slots[wv][P_AL + 1]) << 32) |
+                                __builtin_bit_cast(uint32_t, s_slots[wv][P_AL]);
+          d += bits_to_double(bits);
+        }
+        const uint64_t bits = double_to_bits(d);
+        st_agent(my_part + P_AL, __builtin_bit_cast(float, (uint32_t)bits));
+        st_agent(my_part + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)));
+      }
+      bar_target += (unsigned)a.G;
+      ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag);
+      if (!ok) break;
+      // ---- stage 2: fixed-order sum over the group's workgroups; the prior gradient seeds the sum
+      //      as block 0 does in the reference (mcmc_step_ffma.h:144) ----
+      const float* grp_part = part_base + (size_t)buf * a.G * SLOT;
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        const int p = tid + i * T;
+        if (p < P) {
+          float v = prior_grad(mc, w[i]);
+          for (int r = 0; r < a.G; ++r) v += ld_agent(grp_part + (size_t)r * SLOT + p);
+          g[i] = v;
+        }
+      }
+      if (last) {
+        double d = 0.0;
+        for (int r = 0; r < a.G; ++r) {
+          const float lo = ld_agent(grp_part + (size_t)r * SLOT + P_AL);
+          const float hi = ld_agent(grp_part + (size_t)r * SLOT + P_AL + 1);
+          d += bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
+                              __builtin_bit_cast(uint32_t, lo));
+        }
+        dl_total = d;
+      }
+      buf ^= 1;
+    }
+    if (!ok) break;
+
+    if (trans) {
+      // ---- log accept ratio (kernel_helpers.h:163-175): sum over rows is dl_total; prior and
+      //      kinetic terms summed here in a fixed order ----
+      double part = 0.0;
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        const int p = tid + i * T;
+        if (p < P) {
+          const float dp = prior_logp(mc, w[i]) - prior_logp(mc, wc[i]);
+          const float nm = __builtin_fmaf(eps * 0.5f, g[i], m[i]);  // final half kick
+          float kt = m0[i] * m0[i];
+          kt = __builtin_fmaf(-nm, nm, kt);
+          part += (double)dp + (double)(0.5f * kt);
+        }
+      }
+#pragma unroll
+      for (int msk = 1; msk < 64; msk <<= 1) part += shfl_xor_d(part, msk);
+      __syncthreads();
+      if ((tid & 63) == 0) s_red[wave] = part;
+      __syncthreads();
+      double tot = dl_total;
+#pragma unroll
+      for (int wv = 0; wv < W; ++wv) tot += s_red[wv];
+      const float la = (float)tot;
+      // ---- Metropolis decision (main.h:235-265) ----
+      const float lu = rng_log_uniform(a.seed, (uint32_t)chain, t);
+      const bool acc = lu < la;
+      if (acc) {
+#pragma unroll
+        for (int i = 0; i < PPT; ++i) {
+          wc[i] = w[i];
+          gc[i] = g[i];
+        }
+        sel ^= 1;
+        ++nacc;
+      }
+      // ---- step-size adaptation (main.h:267-276); a non-finite ratio counts as minus infinity ----
+      if ((int)t < a.adapt_steps) {
+        const float laf = (la == la) ? la : -__builtin_inff();
+        const float lmin = laf < 0.0f ? laf : 0.0f;
+        const float adj = lmin < a.log_target ? a.dec_adj : a.inc_adj;
+        eps = eps + eps * adj;
+      }
+      if (rank == 0) {
+        // ---- sample store (main.h:277-283) and traces ----
+        if ((int)t >= a.burn_in && (int)t - a.burn_in < a.n_samples) {
+          float* dst = a.samples + ((size_t)chain * a.n_samples + ((int)t - a.burn_in)) * P;
+#pragma unroll
+          for (int i = 0; i < PPT; ++i) {
+            const int p = tid + i * T;
+            if (p < P) dst[p] = wc[i];
+          }
+        }
+        if (tid == 0 && (int)t < a.trace_len) {
+          a.tr_log_acpt[(size_t)chain * a.trace_len + t] = la;
+          a.tr_accept[(size_t)chain * a.trace_len + t] = acc ? 1 : 0;
+          a.tr_eps[(size_t)chain * a.trace_len + t] = eps;
+        }
+      }
+    }
+  }
+
+  if (!ok) return;
+  // ---- write back ----
+  if (rank == 0) {
+    if (trans) {
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        const int p = tid + i * T;
+        if (p < P) {
+          a.st_w[(size_t)chain * a.st_stride + p] = wc[i];
+          a.st_g[(size_t)chain * a.st_stride + p] = gc[i];
+        }
+      }
+      if (tid == 0) {
+        a.st_eps[chain] = eps;
+        a.st_t[chain] = t0 + a.n_trans;
+        a.st_sel[chain] = sel;
+        a.st_nacc[chain] = nacc;
+      }
+    } else {
+      double psum = 0.0;
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        const int p = tid + i * T;
+        if (p < P) {
+          const size_t o = (size_t)group * a.out_stride + p;
+          const float lp = prior_logp(mc, w[i]);
+          if (a.w_out) a.w_out[o] = w[i];
+          if (a.m_out) a.m_out[o] = m[i];
+          if (a.g_out) a.g_out[o] = g[i];
+          if (a.g_zero) a.g_zero[o] = 0.0f;
+          if (a.prior_out) a.prior_out[o] = lp;
+          psum += (double)lp;
+        }
+      }
+      if (a.sums_out) {
+#pragma unroll
+        for (int msk = 1; msk < 64; msk <<= 1) psum += shfl_xor_d(psum, msk);
+        __syncthreads();
+        if ((tid & 63) == 0) s_red[wave] = psum;
+        __syncthreads();
+        if (tid == 0) {
+          double tot = 0.0;
+#pragma unroll
+          for (int wv = 0; wv < W; ++wv) tot += s_red[wv];
+          a.sums_out[(size_t)group * 2 + 0] = dl_total;
+          a.sums_out[(size_t)group * 2 + 1] = tot;
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host-side launcher
+// ------------------------------------------------------------------------------------------------
+template <class Layer, int LIK, int T>
+static const void* kernel_ptr() {
+  return reinterpret_cast<const void*>(&hmc_kernel<Layer, LIK, T>);
+}
+
+const void* hmc_kernel_for(int d0, int d1, int layer, int lik, int threads) {
+  if (d0 != 22 || d1 != 40) return nullptr;
+  using M = MfmaLayer<22, 40>;
+  using F = FfmaLayer<22, 40>;
+  if (layer == 0) {
+    if (threads == 512) return lik == 0 ? kernel_ptr<M, 0, 512>() : kernel_ptr<M, 1, 512>();
+    if (threads == 256) return lik == 0 ? kernel_ptr<M, 0, 256>() : kernel_ptr<M, 1, 256>();
+  } else if (layer == 1) {
+    if (threads == 256) return lik == 0 ? kernel_ptr<F, 0, 256>() : kernel_ptr<F, 1, 256>();
+  }
+  return nullptr;
+}
+
+hipError_t launch_hmc_kernel(const void* kernel, const KArgs& args, int workgroups, int threads,
+                             hipStream_t stream) {
+  KArgs a = args;
+  void* params[] = {&a};
+  return hipLaunchKernel(kernel, dim3(workgroups), dim3(threads), params, 0, stream);
+}
+
+}  // namespace bnn

@@ -1,0 +1,211 @@
+// Host driver of the MI355X HMC sampler: the three phases of the reference's mcmc::main_loop
+// (include/mcmc/main.h:117-308) -- init, run N samples, dump the chain -- on top of the C ABI in
+// include/bnn_hmc.h.  Plain C++, no GPU code here.
+//
+//   bnn_hmc_main [--windows W] [--chains C] [--samples S] [--burn-in B] [--leapfrog L] [--rows N]
+//                [--lik student_t|gaussian] [--layer mfma|ffma] [--cus-per-chain G] [--wgs-per-cu K]
+//                [--seed S] [--data FILE] [--dump FILE]
+//
+// Without --data every window is filled with the synthetic recipe (features ~ N(0,1), targets from
+// a random teacher MLP plus noise).  With --data the reference's text format is read
+// (include/mcmc/io.h:43-86) into window 0 and the features are scaled by 0.001 (main.h:162-164).
+#include <chrono>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "bnn_hmc.h"
+
+namespace {
+
+struct Options {
+  int windows = 1, chains = 1, samples = 800, burn_in = 100, leapfrog = 1000, rows = 58368;
+  int lik = BNNHMC_LIK_STUDENT_T, layer = BNNHMC_LAYER_MFMA, cus_per_chain = 0, wgs_per_cu = 0;
+  unsigned seed = 0;
+  std::string data, dump;
+};
+
+void die(const char* what) {
+  std::fprintf(stderr, "error: %s: %s\n", what, bnnhmc_last_error());
+  std::exit(1);
+}
+#define CHECK(call)            \
+  do {                         \
+    if ((call) != BNNHMC_OK) die(#call); \
+  } while (0)
+
+bool parse(int argc, char** argv, Options& o) {
+  for (int i = 1; i < argc; ++i) {
+    std::string a = argv[i];
+    auto next = [&]() -> const char* { return i + 1 < argc ? argv[++i] : ""; };
+    if (a == "--windows") o.windows = std::atoi(next());
+    else if (a == "--chains") o.chains = std::atoi(next());
+    else if (a == "--samples") o.samples = std::atoi(next());
+    else if (a == "--burn-in") o.burn_in = std::atoi(next());
+    else if (a == "--leapfrog") o.leapfrog = std::atoi(next());
+    else if (a == "--rows") o.rows = std::atoi(next());
+    else if (a == "--seed") o.seed = (unsigned)std::strtoul(next(), nullptr, 10);
+    else if (a == "--cus-per-chain") o.cus_per_chain = std::atoi(next());
+    else if (a == "--wgs-per-cu") o.wgs_per_cu = std::atoi(next());
+    else if (a == "--lik") o.lik = std::string(next()) == "gaussian" ? BNNHMC_LIK_GAUSSIAN : BNNHMC_LIK_STUDENT_T;
+    else if (a == "--layer") o.layer = std::string(next()) == "ffma" ? BNNHMC_LAYER_FFMA : BNNHMC_LAYER_MFMA;
+    else if (a == "--data") o.data = next();
+    else if (a == "--dump") o.dump = next();
+    else {
+      std::fprintf(stderr, "unknown option %s\n", a.c_str());
+      return false;
+    }
+  }
+  return true;
+}
+
+// the reference's dataset format (include/mcmc/io.h:43-86): one header line of 149 tokens, then per
+// row 149 columns of which the first 2 are skipped, the next is the label and the next 22 the features
+bool read_reference_data(const std::string& path, int rows, std::vector<float>& x, std::vector<float>& y) {
+  const int total_cols = 149, skip = 2, d0 = 22;
+  FILE* fp = std::fopen(path.c_str(), "r");
+  if (!fp) return false;
+  char buf[256];
+  for (int j = 0; j < total_cols; ++j)
+    if (std::fscanf(fp, "%255s", buf) == EOF) break;
+  x.assign((size_t)rows * d0, 0.0f);
+  y.assign(rows, 0.0f);
+  for (int i = 0; i < rows; ++i) {
+    for (int j = 0; j < total_cols; ++j) {
+      if (std::fscanf(fp, "%255s", buf) == EOF) {
+        std::fclose(fp);
+        return false;
+      }
+      if (j < skip || j >= skip + 1 + d0) continue;
+      const float v = std::strtof(buf, nullptr);
+      if (j == skip) y[i] = v;
+      else x[(size_t)i * d0 + (j - skip - 1)] = v;
+    }
+  }
+  std::fclose(fp);
+  return true;
+}
+
+// shape / min / max / mean summary the reference prints for a matrix (utils_matrix.h:160-178)
+void print_stats(const char* name, const float* d, size_t rows, size_t cols) {
+  float mn = INFINITY, mx = -INFINITY, mean = 0.0f;
+  const size_t n = rows * cols;
+  for (size_t i = 0; i < n; ++i) {
+    mean += d[i] / (float)n;
+    if (d[i] > mx) mx = d[i];
+    if (d[i] < mn) mn = d[i];
+  }
+  std::printf("%s: Shape: %zu x %zu, word: 4, min: %g, max: %g, mean: %g\n", name, rows, cols, mn, mx, mean);
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+  Options o;
+  if (!parse(argc, argv, o)) return 2;
+
+  // ------------------------------------------------------------------ init (main.h:120-202)
+  bnnhmc_model model;
+  bnnhmc_default_model(&model);
+  model.n = o.rows;
+  model.lik_kind = o.lik;
+  if (o.lik == BNNHMC_LIK_GAUSSIAN) {  // the benchmark configs: sigma 0.01, prior N(0, 0.1^2)
+    model.lik_scale = 0.01;
+    model.prior_scale = 0.1;
+  }
+  bnnhmc_hmc hmc;
+  bnnhmc_default_hmc(&hmc);
+  hmc.n_samples = o.samples;
+  hmc.burn_in = o.burn_in;
+  hmc.adapt_steps = o.burn_in;
+  hmc.leapfrog_steps = o.leapfrog;
+  hmc.seed = o.seed;
+  bnnhmc_launch launch;
+  bnnhmc_default_launch(&launch);
+  launch.layer = o.layer;
+  if (o.cus_per_chain > 0) launch.cus_per_chain = o.cus_per_chain;
+  if (o.wgs_per_cu > 0) launch.wgs_per_cu = o.wgs_per_cu;
+
+  int n_dev = 0, cus = 0;
+  char arch[64];
+  CHECK(bnnhmc_device_info(&n_dev, &cus, arch, sizeof(arch)));
+  std::printf("Device 0: %s, %d compute units. %d window(s) x %d chain(s), %d workgroups per chain, %s layer.\n",
+              arch, cus, o.windows, o.chains, launch.cus_per_chain,
+              o.layer == BNNHMC_LAYER_FFMA ? "FFMA" : "MFMA");
+
+  bnnhmc_sampler* s = nullptr;
+  CHECK(bnnhmc_create(&model, &hmc, &launch, o.windows, o.chains, &s));
+  const int P = bnnhmc_num_params(model.d0, model.d1);
+  if (!o.data.empty()) {
+    std::vector<float> x, y;
+    std::printf("Reading dataset...\n");
+    if (!read_reference_data(o.data, model.n, x, y)) {
+      std::fprintf(stderr, "Error: failed to read file '%s'!\n", o.data.c_str());
+      return 1;
+    }
+    std::printf("Dataset read successfully\n");
+    print_stats("Data", x.data(), model.n, model.d0);
+    print_stats("Labels", y.data(), model.n, 1);
+    for (float& v : x) v *= 0.001f;  // main.h:162-164
+    for (int w = 0; w < o.windows; ++w) CHECK(bnnhmc_set_window_data(s, w, x.data(), y.data()));
+  } else {
+    for (int w = 0; w < o.windows; ++w) CHECK(bnnhmc_generate_window(s, w, 0.1f, 0.01f, nullptr));
+    std::vector<float> x((size_t)model.n * model.d0), y(model.n);
+    CHECK(bnnhmc_get_window_data(s, 0, x.data(), y.data()));
+    print_stats("Data", x.data(), model.n, model.d0);
+    print_stats("Labels", y.data(), model.n, 1);
+  }
+
+  const auto t_start = std::chrono::high_resolution_clock::now();  // main.h:187-189
+  CHECK(bnnhmc_init_chains(s, nullptr));
+
+  // ------------------------------------------------------------------ run (main.h:204-287)
+  const int total = hmc.burn_in + hmc.n_samples, every = 10;
+  for (int done = 0; done < total; done += every) {
+    CHECK(bnnhmc_run(s, std::min(every, total - done)));
+    std::printf(".");
+    std::fflush(stdout);
+  }
+  std::printf("\n");
+  const auto t_end = std::chrono::high_resolution_clock::now();  // main.h:293
+
+  // ------------------------------------------------------------------ dump (main.h:295-307)
+  std::vector<float> samples((size_t)hmc.n_samples * P);
+  FILE* out = o.dump.empty() ? nullptr : std::fopen(o.dump.c_str(), "wb");
+  for (int c = 0; c < o.windows * o.chains; ++c) {
+    int stored = 0;
+    CHECK(bnnhmc_get_samples(s, c, samples.data(), &stored));
+    if (c == 0) print_stats("Final samples", samples.data(), stored, P);
+    if (out) std::fwrite(samples.data(), sizeof(float), (size_t)stored * P, out);
+  }
+  if (out) {
+    std::fclose(out);
+    std::printf("Wrote %d chain(s) x %d samples x %d floats to %s\n", o.windows * o.chains,
+                hmc.n_samples, P, o.dump.c_str());
+  }
+  double l1 = 0, l2 = 0, fl = 0;
+  if (hmc.n_samples > 0) {
+    CHECK(bnnhmc_final_loss(s, 0, &l1, &l2, &fl));
+    std::printf("Final loss1: %g, loss2: %g, full loss: %g\n", l1, l2, fl);
+  }
+  float eps = 0;
+  int n_acc = 0, n_done = 0;
+  CHECK(bnnhmc_get_chain_state(s, 0, nullptr, nullptr, &eps, &n_done, &n_acc));
+  double kernel_ms = 0;
+  long launches = 0, evals = 0;
+  int wgs = 0;
+  CHECK(bnnhmc_get_timing(s, &kernel_ms, &launches, &evals, &wgs));
+  const double t_ms = std::chrono::duration<double, std::milli>(t_end - t_start).count();
+  std::printf("Chain 0: %d/%d transitions accepted, final eps %g\n", n_acc, n_done, eps);
+  std::printf("MCMC (%d burn in, %d sample steps, %d leap-frog steps) done in %.0fms; %ld gradient "
+              "evaluations, %.1f evals/s (device %.0fms).\n",
+              hmc.burn_in, hmc.n_samples, hmc.leapfrog_steps, t_ms, evals, evals / (t_ms * 1e-3),
+              kernel_ms);
+  if (o.windows * o.chains == 1)
+    std::printf("Expected time for 200 sequential passes: %.3fh. Good bye!\n", 200 * (t_ms / 3600000.0));
+  CHECK(bnnhmc_destroy(s));
+  return 0;
+}

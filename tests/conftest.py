@@ -18,3 +18,15 @@ def orc():
     import orc_binding
 
     return orc_binding.load()
+
+
+@pytest.fixture(scope="session")
+def pkg():
+    import __graft_entry__ as ge
+
+    return ge.load_package()
+
+
+@pytest.fixture(scope="session")
+def lib(pkg):
+    return pkg.load()

@@ -1,0 +1,108 @@
+"""CPU-only checks of the shipped library: it loads, exports the whole C ABI, its host-side
+generator and RNG agree bit for bit with the oracle's independent restatement, and its error paths
+return codes instead of aborting.  No compute is launched here."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import orc_binding as ob
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(pkg, lib):
+    header = open(os.path.join(ROOT, "include", "bnn_hmc.h")).read()
+    declared = set(re.findall(r"\b(bnnhmc_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    assert declared == set(pkg.EXPORTS)
+    for name in declared:
+        assert hasattr(lib.c, name), name
+
+
+def test_struct_layouts_match_header(pkg):
+    assert C.sizeof(pkg.Model) == 4 * 4 + 3 * 8
+    assert C.sizeof(pkg.Hmc) == 4 * 4 + 4 * 4 + 4
+    assert C.sizeof(pkg.Launch) == 5 * 4
+
+
+def test_defaults_are_the_reference_constants(lib):
+    m = lib.default_model()
+    assert (m.d0, m.d1, m.n) == (22, 40, 58368)                      # global_params.h:56, 61
+    assert (m.lik_kind, m.lik_scale, m.lik_df, m.prior_scale) == (0, 100.0, 2.2, 200.0)
+    h = lib.default_hmc()
+    assert (h.leapfrog_steps, h.burn_in, h.n_samples, h.adapt_steps) == (1000, 100, 800, 100)
+    assert h.eps0 == np.float32(0.01) and h.target_rate == np.float32(0.2)
+    assert h.decrement == np.float32(0.1) and h.increment == np.float32(0.01)
+    assert lib.num_params(22, 40) == 961
+
+
+def test_host_rng_matches_oracle_bit_for_bit(lib, orc):
+    for (seed, id_, stream, t, idx) in [(0, 0, 3, 0, 0), (7, 199, 3, 899, 960), (1, 2, 0, 0, 1284095),
+                                        (123456789, 799, 4, 1699, 0), (5, 6, 2, 0, 58367)]:
+        assert lib.rng_word(seed, id_, stream, t, idx) == orc.rng_word(seed, id_, stream, t, idx)
+        a = np.float32(lib.rng_normal(seed, id_, stream, t, idx))
+        b = np.float32(orc.normal(seed, id_, stream, t, idx))
+        assert a.tobytes() == b.tobytes()
+    for t in range(200):
+        a = np.float32(lib.rng_log_uniform(3, 4, t))
+        b = np.float32(orc.log_uniform(3, 4, t))
+        assert a.tobytes() == b.tobytes()
+    mom = orc.momentum(11, 5, 17, 961)
+    mine = np.array([lib.rng_normal(11, 5, 3, 17, p) for p in range(961)], np.float32)
+    assert mine.tobytes() == mom.tobytes()
+
+
+def test_host_generator_matches_oracle_bit_for_bit(lib, orc):
+    for (seed, window, n) in [(0, 0, 300), (0, 7, 64), (9, 199, 33)]:
+        X, y, th = lib.generate_window_host(seed, window, n)
+        Xo, yo, tho = orc.gen_window(seed, window, n)
+        assert X.tobytes() == Xo.tobytes()
+        assert th.tobytes() == tho.tobytes()
+        assert y.tobytes() == yo.tobytes()
+
+
+def test_error_codes_without_launching(pkg, lib):
+    m = lib.default_model()
+    h = lib.default_hmc()
+    l = lib.default_launch()
+    hnd = C.c_void_p()
+    # unsupported shape
+    bad = lib.default_model(d0=23)
+    rc = lib.c.bnnhmc_create(C.byref(bad), C.byref(h), C.byref(l), 1, 1, C.byref(hnd))
+    assert rc == pkg.ERR_INVALID and b"unsupported layer sizes" in lib.c.bnnhmc_last_error()
+    for kw in (dict(n=0), dict(lik_kind=5), dict(lik_scale=0.0), dict(prior_scale=-1.0), dict(lik_df=0.0)):
+        bad = lib.default_model(**kw)
+        assert lib.c.bnnhmc_create(C.byref(bad), C.byref(h), C.byref(l), 1, 1, C.byref(hnd)) == pkg.ERR_INVALID
+    assert lib.c.bnnhmc_create(None, C.byref(h), C.byref(l), 1, 1, C.byref(hnd)) == pkg.ERR_INVALID
+    assert lib.c.bnnhmc_create(C.byref(m), None, C.byref(l), 1, 1, C.byref(hnd)) == pkg.ERR_INVALID
+    assert lib.c.bnnhmc_create(C.byref(m), C.byref(h), C.byref(l), 0, 1, C.byref(hnd)) == pkg.ERR_INVALID
+    assert lib.c.bnnhmc_create(C.byref(m), C.byref(h), C.byref(l), 1, 1, None) == pkg.ERR_INVALID
+    badh = lib.default_hmc(leapfrog_steps=0)
+    assert lib.c.bnnhmc_create(C.byref(m), C.byref(badh), C.byref(l), 1, 1, C.byref(hnd)) == pkg.ERR_INVALID
+    # null handles
+    assert lib.c.bnnhmc_run(None, 1) == pkg.ERR_INVALID
+    assert lib.c.bnnhmc_init_chains(None, None) == pkg.ERR_INVALID
+    assert lib.c.bnnhmc_get_samples(None, 0, None, None) == pkg.ERR_INVALID
+    assert lib.c.bnnhmc_destroy(None) == pkg.OK
+    # operator level: null pointers and bad sizes are rejected before anything is launched
+    rc = lib.c.bnnhmc_mcmc_step(C.byref(m), C.byref(l), None, None, None, None, None, None, None, None,
+                                None, None, None, C.c_size_t(0), C.c_float(0.01), 1, None)
+    assert rc == pkg.ERR_INVALID
+    assert lib.c.bnnhmc_log_acpt(-1, 0, None, None, None, None, None, C.c_float(0), None, None, None) == pkg.ERR_INVALID
+    assert lib.c.bnnhmc_sample_momentum(0, 0, 0, -1, None, None, None) == pkg.ERR_INVALID
+    assert lib.c.bnnhmc_get_loss_values(None, 1, 1, None, None, None) == pkg.ERR_INVALID
+    assert lib.step_workspace_bytes(m, l) >= 2 * 32 * 961 * 4
+
+
+def test_no_device_is_reported_not_faked(pkg, lib):
+    rc, n_dev, cus, arch = lib.device_info()
+    if n_dev > 0:
+        pytest.skip("a GPU is visible")
+    assert rc == pkg.ERR_NO_DEVICE
+    m, h, l = lib.default_model(n=64), lib.default_hmc(), lib.default_launch()
+    hnd = C.c_void_p()
+    assert lib.c.bnnhmc_create(C.byref(m), C.byref(h), C.byref(l), 1, 1, C.byref(hnd)) == pkg.ERR_NO_DEVICE
+    assert not hnd.value

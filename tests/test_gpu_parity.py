@@ -1,0 +1,323 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle on the same seeded
+inputs.  Tolerances (FP32 path): gradients and energies within 1e-5 relative to the largest gradient
+component / the energy scale; RNG streams and decisions bit-exact."""
+import math
+import sys
+
+import numpy as np
+import pytest
+
+import orc_binding as ob
+from hipmem import DevBuf, synchronize
+
+pytestmark = pytest.mark.gpu
+
+D0, D1, P = 22, 40, 961
+RTOL = 1e-5
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def models(pkg, lib, kind, n):
+    """(library model, oracle model, generator arguments): the reference's Student-t setup and the
+    benchmark's Gaussian setup.  Teacher weights are sized so that the hidden pre-activations are
+    O(1): with saturated tanh units the factor 1 - h^2 cancels catastrophically in FP32 (in the
+    reference's formulation as much as here) and no FP32 implementation agrees to 1e-5."""
+    if kind == "t":
+        return (lib.default_model(n=n), ob.Model(D0, D1, n, ob.LIK_STUDENT_T, 100.0, 2.2, 200.0),
+                dict(teacher_scale=0.3, noise_sigma=5.0))
+    if kind == "t_stiff":  # a Student-t posterior tight enough that HMC rejects part of the time
+        return (lib.default_model(n=n, lik_scale=0.5, prior_scale=2.0),
+                ob.Model(D0, D1, n, ob.LIK_STUDENT_T, 0.5, 2.2, 2.0), dict(teacher_scale=0.3, noise_sigma=0.5))
+    return (lib.default_model(n=n, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1),
+            ob.Model(D0, D1, n, ob.LIK_GAUSSIAN, 0.01, 0.0, 0.1), dict(teacher_scale=0.1, noise_sigma=0.01))
+
+
+def close_grad(a, b, what, rtol=RTOL):
+    scale = float(np.abs(b).max())
+    err = float(np.abs(a.astype(np.float64) - b).max())
+    assert err <= rtol * scale + 1e-30, "%s: max abs err %.3e vs scale %.3e" % (what, err, scale)
+
+
+# ------------------------------------------------------------------------------------------------
+# RNG: device stream == host mirror == oracle, bit for bit
+# ------------------------------------------------------------------------------------------------
+def test_device_momentum_stream_is_bit_exact(lib, orc):
+    say("momentum stream")
+    for (seed, chain, t) in [(0, 0, 0), (7, 199, 899), (123, 3, 57)]:
+        a = DevBuf.full(P + 1, np.nan)
+        b = DevBuf.full(P + 1, np.nan)
+        lib.sample_momentum(seed, chain, t, P + 1, a.ptr, b.ptr, 0)
+        synchronize()
+        ref = orc.momentum(seed, chain, t, P + 1)
+        assert a.numpy(P + 1).tobytes() == ref.tobytes()
+        assert b.numpy(P + 1).tobytes() == ref.tobytes()
+
+
+# ------------------------------------------------------------------------------------------------
+# log-posterior / gradient (the fused forward + backward + reduction)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("layer", ["mfma", "ffma"])
+@pytest.mark.parametrize("kind", ["t", "gauss"])
+@pytest.mark.parametrize("n,G", [(1, 1), (3, 2), (16, 1), (17, 4), (100, 3), (1000, 8), (4101, 32),
+                                 (58368, 32)])
+def test_eval_matches_oracle(pkg, lib, orc, layer, kind, n, G):
+    say("eval layer=%s lik=%s n=%d G=%d" % (layer, kind, n, G))
+    model, om, gen = models(pkg, lib, kind, n)
+    launch = lib.default_launch(layer=pkg.LAYER_MFMA if layer == "mfma" else pkg.LAYER_FFMA,
+                                cus_per_chain=G)
+    s = lib.create(model, lib.default_hmc(seed=n), launch, 1, 1)
+    th = s.generate_window(0, **gen)
+    X, y = s.get_window_data(0)
+    Xo, yo, tho = orc.gen_window(n, 0, n, **gen)
+    assert X.tobytes() == Xo.tobytes() and y.tobytes() == yo.tobytes()
+    rng = np.random.default_rng(n)
+    for w in (np.zeros(P, np.float32), (th * 0.7 + rng.normal(0, 0.02 * gen["teacher_scale"], P)).astype(np.float32)):
+        ell, prior, grad = s.eval(0, w)
+        ell_o, prior_o, grad_o, _ = orc.eval_f32(om, X, y, w)
+        _, _, grad64 = orc.eval_f64(om, X, y, w.astype(np.float64))
+        close_grad(grad, grad_o, "grad vs f32 oracle")
+        close_grad(grad, grad64, "grad vs f64 oracle", rtol=2e-5)
+        np.testing.assert_allclose(ell, ell_o, rtol=RTOL, atol=RTOL * max(1.0, float(np.abs(ell_o).max())))
+        assert prior.tobytes() == prior_o.tobytes()
+        # potential energy
+        U, Uo = -(ell.sum(dtype=np.float64) + prior.sum(dtype=np.float64)), -(
+            ell_o.sum(dtype=np.float64) + prior_o.sum(dtype=np.float64))
+        assert abs(U - Uo) <= RTOL * abs(Uo)
+    s.close()
+
+
+def test_eval_is_deterministic_and_layout_agnostic(pkg, lib, orc):
+    n = 5000
+    model, om, gen = models(pkg, lib, "t", n)
+    outs = {}
+    for G in (1, 4, 32):
+        for rep in range(2):
+            s = lib.create(model, lib.default_hmc(seed=3), lib.default_launch(cus_per_chain=G), 1, 1)
+            th = s.generate_window(0, **gen)
+            _, _, grad = s.eval(0, th)
+            s.close()
+            if rep == 0:
+                outs[G] = grad
+            else:
+                assert grad.tobytes() == outs[G].tobytes(), "two runs differ at G=%d" % G
+    close_grad(outs[1], outs[32].astype(np.float64), "G=1 vs G=32", rtol=3e-6)
+    close_grad(outs[4], outs[32].astype(np.float64), "G=4 vs G=32", rtol=3e-6)
+
+
+# ------------------------------------------------------------------------------------------------
+# the step operator through caller-owned device buffers
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("layer", ["mfma", "ffma"])
+@pytest.mark.parametrize("kind,n,L,eps,G", [("t", 777, 1, 0.01, 4), ("t", 2048, 2, 0.01, 8),
+                                            ("t", 1500, 25, 0.01, 32), ("gauss", 999, 10, 1e-5, 5),
+                                            ("gauss", 4096, 40, 2e-5, 32)])
+def test_mcmc_step_operator_matches_oracle(pkg, lib, orc, layer, kind, n, L, eps, G):
+    say("mcmc_step layer=%s lik=%s n=%d L=%d G=%d" % (layer, kind, n, L, G))
+    model, om, gen = models(pkg, lib, kind, n)
+    launch = lib.default_launch(layer=pkg.LAYER_MFMA if layer == "mfma" else pkg.LAYER_FFMA,
+                                cus_per_chain=G)
+    X, y, th = orc.gen_window(5, 1, n, **gen)
+    rng = np.random.default_rng(n + L)
+    w0 = (th * 0.8).astype(np.float32)
+    m0 = rng.normal(0, 1, P).astype(np.float32)
+    g0 = orc.eval_f32(om, X, y, w0)[2]
+    dev = DevBuf.from_numpy
+    dX, dy, dw0, dm0, dg0 = dev(X), dev(y), dev(w0), dev(m0), dev(g0)
+    dw1, dm1, dg1, dgn = (DevBuf.full(P, np.nan) for _ in range(4))
+    dloss = DevBuf.full(n + P, np.nan)
+    wsb = lib.step_workspace_bytes(model, launch)
+    ws = DevBuf.full(wsb // 4 + 16, 0, np.int32)
+    st = 0  # the default stream
+    lib.mcmc_step(model, launch, dX.ptr, dy.ptr, dw0.ptr, dw1.ptr, dm0.ptr, dm1.ptr, dg0.ptr, dg1.ptr,
+                  dgn.ptr, dloss.ptr, ws.ptr, wsb, eps, L, st)
+    lib.step_check(model, launch, ws.ptr, st)
+    w1, m1, g1 = dw1.numpy(P), dm1.numpy(P), dg1.numpy(P)
+    loss = dloss.numpy(n + P)
+    w1o, m1o, g1o, losso = orc.mcmc_step(om, X, y, w0, m0, g0, eps, L)
+    assert np.all(dgn.numpy(P) == 0)                           # grad_next is zeroed
+    # positions / momenta agree to FP32 rounding accumulated over L steps
+    np.testing.assert_allclose(w1, w1o, rtol=0, atol=1e-6 * L * max(1.0, float(np.abs(w1o).max())))
+    np.testing.assert_allclose(m1, m1o, rtol=0, atol=3e-6 * L * max(1.0, float(np.abs(m1o).max())))
+    close_grad(g1, g1o.astype(np.float64), "grad_cur", rtol=RTOL * max(1, L // 4))
+    np.testing.assert_allclose(loss[:n], losso[:n], rtol=1e-5 * max(1, L // 4),
+                               atol=1e-5 * max(1, L // 4) * max(1.0, float(np.abs(losso[:n]).max())))
+    np.testing.assert_allclose(loss[n:], losso[n:], rtol=1e-6, atol=1e-6)
+    # the log accept ratio of this trajectory (log_acpt_prec) and the loss sums
+    ell0, prior0, _, _ = orc.eval_f32(om, X, y, w0)
+    prev_loss = np.concatenate([ell0, prior0])
+    dprev = dev(prev_loss)
+    dout = DevBuf.full(1, 0.0)
+    la = lib.log_acpt(n + P, P, dprev.ptr, dloss.ptr, dm0.ptr, dm1.ptr, dg1.ptr, eps, dout.ptr, st)
+    la_same_inputs = orc.log_acpt(prev_loss, loss, m0, m1, g1, eps)
+    assert la == pytest.approx(la_same_inputs, rel=1e-6, abs=1e-6)
+    assert float(dout.numpy(1)[0]) == la
+    l1, l2 = lib.get_loss_values(dloss.ptr, n, P, st)
+    assert l1 == pytest.approx(float(loss[:n].sum(dtype=np.float64)), rel=1e-6)
+    assert l2 == pytest.approx(float(loss[n:].sum(dtype=np.float64)), rel=1e-6)
+
+
+def test_mcmc_step_accepts_unaligned_caller_buffers(pkg, lib, orc):
+    n, L, eps = 333, 3, 0.01
+    model, om, gen = models(pkg, lib, "t", n)
+    launch = lib.default_launch(cus_per_chain=2)
+    X, y, th = orc.gen_window(6, 0, n, **gen)
+    w0 = th.astype(np.float32)
+    m0 = np.ones(P, np.float32)
+    g0 = orc.eval_f32(om, X, y, w0)[2]
+
+    bx = DevBuf.from_numpy(X, offset_bytes=4)    # 4-byte aligned only
+    by = DevBuf.from_numpy(y, offset_bytes=12)
+    bufs = [DevBuf.from_numpy(a) for a in (w0, m0, g0)]
+    outs = [DevBuf.full(P, 0.0) for _ in range(4)]
+    dloss = DevBuf.full(n + P, 0.0)
+    wsb = lib.step_workspace_bytes(model, launch)
+    ws = DevBuf.full(wsb // 4 + 16, 0, np.int32)
+    st = 0
+    lib.mcmc_step(model, launch, bx.data_ptr, by.data_ptr, bufs[0].ptr, outs[0].ptr, bufs[1].ptr,
+                  outs[1].ptr, bufs[2].ptr, outs[2].ptr, outs[3].ptr, dloss.ptr, ws.ptr, wsb, eps, L, st)
+    lib.step_check(model, launch, ws.ptr, st)
+    w1o, m1o, g1o, losso = orc.mcmc_step(om, X, y, w0, m0, g0, eps, L)
+    close_grad(outs[2].numpy(P), g1o.astype(np.float64), "grad_cur (unaligned)")
+    np.testing.assert_allclose(outs[0].numpy(P), w1o, atol=1e-5)
+
+
+# ------------------------------------------------------------------------------------------------
+# whole transitions on the device: RNG, accept, adaptation, sample store
+# ------------------------------------------------------------------------------------------------
+def _run_pair(pkg, lib, orc, kind, n, L, burn, keep, eps0, G, layer="mfma", seed=21, tpl=5):
+    model, om, gen = models(pkg, lib, kind, n)
+    hmc = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=eps0, seed=seed)
+    launch = lib.default_launch(layer=pkg.LAYER_MFMA if layer == "mfma" else pkg.LAYER_FFMA,
+                                cus_per_chain=G, transitions_per_launch=tpl)
+    s = lib.create(model, hmc, launch, 1, 1)
+    s.generate_window(0, **gen)
+    X, y = s.get_window_data(0)
+    s.init_chains(None)
+    s.run(burn + keep)
+    out = dict(samples=s.get_samples(0), state=s.get_chain_state(0), traces=s.get_traces(0),
+               final_loss=s.final_loss(0) if keep else None, timing=s.timing())
+    s.close()
+    oh = ob.Hmc(L, burn, keep, burn, eps0, 0.2, 0.1, 0.01, seed, 0)
+    ref = orc.run_chain(om, oh, X, y)
+    return out, ref, (om, X, y)
+
+
+@pytest.mark.parametrize("layer", ["mfma", "ffma"])
+def test_transitions_match_oracle_decisions(pkg, lib, orc, layer):
+    say("transitions layer=%s" % layer)
+    n, L, burn, keep = 2048, 20, 30, 30
+    out, ref, (om, X, y) = _run_pair(pkg, lib, orc, "t_stiff", n, L, burn, keep, 0.01, 8, layer=layer)
+    T = burn + keep
+    tr = out["traces"]
+    assert len(tr["accept"]) == T
+    la, la_o = tr["log_acpt"], ref["log_acpt"]
+    # identical accept/reject decisions over the first 50 transitions, same RNG stream
+    margin = np.abs(np.array([orc.log_uniform(21, 0, t) for t in range(T)]) - la_o)
+    assert margin[:50].min() > 1e-3, "test inputs put a decision on a knife edge"
+    assert np.array_equal(tr["accept"][:50], ref["accept"][:50])
+    assert np.array_equal(tr["accept"], ref["accept"])
+    assert 0 < ref["accept"].sum() < T
+    np.testing.assert_allclose(la, la_o, rtol=2e-3, atol=5e-3)
+    assert tr["eps"].tobytes() == ref["eps"].tobytes()          # adaptation follows decisions exactly
+    assert out["state"]["n_accepted"] == ref["n_accept"]
+    assert out["state"]["transitions_done"] == T
+    assert out["state"]["eps"] == ref["final_eps"]
+    np.testing.assert_allclose(out["samples"], ref["samples"], rtol=0, atol=2e-4 * max(1.0, float(np.abs(ref["samples"]).max())))
+    np.testing.assert_allclose(out["state"]["w"], ref["final_w"], rtol=0, atol=2e-4 * max(1.0, float(np.abs(ref["final_w"]).max())))
+    # sample store: rejected transitions repeat the previous row
+    for t in range(burn + 1, T):
+        if not tr["accept"][t]:
+            assert np.array_equal(out["samples"][t - burn], out["samples"][t - burn - 1])
+    l1, l2, fl = out["final_loss"]
+    o1, o2, ofl = orc.final_loss(om, X, y, out["samples"])
+    assert l1 == pytest.approx(o1, rel=1e-5) and l2 == pytest.approx(o2, rel=1e-6)
+    assert fl == pytest.approx(ofl, rel=1e-5)
+    assert out["timing"]["grad_evals"] == T * L
+
+
+def test_divergent_trajectories_reject_and_restore(pkg, lib, orc):
+    # the benchmark's stiff Gaussian posterior with the reference's eps0 = 0.01 diverges to inf/NaN
+    # until adaptation has shrunk eps: every such transition must reject and leave the state alone
+    n, L, burn, keep = 1024, 30, 40, 5
+    out, ref, _ = _run_pair(pkg, lib, orc, "gauss", n, L, burn, keep, 0.01, 4)
+    tr = out["traces"]
+    assert not np.isfinite(tr["log_acpt"][0]) or tr["log_acpt"][0] < -1e6
+    assert tr["accept"][0] == 0
+    assert np.array_equal(tr["accept"], ref["accept"])
+    assert tr["eps"].tobytes() == ref["eps"].tobytes()
+    assert np.all(np.isfinite(out["state"]["w"]))
+    assert tr["eps"][-1] < 0.01 * 0.5
+
+
+def test_runs_are_bit_reproducible_and_chunking_is_invisible(pkg, lib, orc):
+    n, L, burn, keep = 1500, 12, 6, 10
+    a, _, _ = _run_pair(pkg, lib, orc, "t", n, L, burn, keep, 0.02, 8, tpl=5)
+    b, _, _ = _run_pair(pkg, lib, orc, "t", n, L, burn, keep, 0.02, 8, tpl=5)
+    c, _, _ = _run_pair(pkg, lib, orc, "t", n, L, burn, keep, 0.02, 8, tpl=1)
+    assert a["samples"].tobytes() == b["samples"].tobytes()
+    assert a["samples"].tobytes() == c["samples"].tobytes()
+    assert a["traces"]["log_acpt"].tobytes() == c["traces"]["log_acpt"].tobytes()
+
+
+def test_many_windows_and_chains_are_independent(pkg, lib, orc):
+    # 5 windows x 2 chains with more chain groups than fit at once at G = 64 -> several rounds
+    n, L, burn, keep = 640, 6, 4, 6
+    model, om, gen = models(pkg, lib, "t", n)
+    hmc = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=0.02, seed=9)
+    launch = lib.default_launch(cus_per_chain=64, transitions_per_launch=4)
+    s = lib.create(model, hmc, launch, 5, 2)
+    for w in range(5):
+        s.generate_window(w, **gen)
+    s.init_chains(None)
+    s.run(burn + keep)
+    for chain in (0, 3, 9):
+        X, y = s.get_window_data(chain // 2)
+        oh = ob.Hmc(L, burn, keep, burn, 0.02, 0.2, 0.1, 0.01, 9, chain)
+        ref = orc.run_chain(om, oh, X, y)
+        tr = s.get_traces(chain)
+        assert np.array_equal(tr["accept"], ref["accept"]), chain
+        np.testing.assert_allclose(s.get_samples(chain), ref["samples"], atol=2e-4 * float(np.abs(ref["samples"]).max() + 1))
+    assert not np.array_equal(s.get_samples(0), s.get_samples(1))   # chains of one window differ
+    assert s.timing()["grad_evals"] == 10 * (burn + keep) * L
+    s.close()
+
+
+# ------------------------------------------------------------------------------------------------
+# size-independent properties at the full 58368-row size
+# ------------------------------------------------------------------------------------------------
+def test_full_size_properties(pkg, lib, orc):
+    n = 58368
+    model, om, gen = models(pkg, lib, "t", n)
+    s = lib.create(model, lib.default_hmc(seed=0), lib.default_launch(), 1, 1)
+    th = s.generate_window(0, **gen)
+    X, y = s.get_window_data(0)
+    # known answer at w = 0 (the reference's initial state): only b2 has a gradient
+    ell, prior, grad = s.eval(0, np.zeros(P, np.float32))
+    assert np.all(grad[:P - 1] == 0)
+    d = y.astype(np.float64) / 100.0
+    assert grad[-1] == pytest.approx(np.sum(d * 3.2 / 100.0 / (d * d + 2.2)), rel=1e-6)
+    assert prior.sum(dtype=np.float64) == pytest.approx(-961 * 6.21725589975271, rel=1e-7)
+    # additivity over rows: gradient of the first half + second half - prior = whole
+    w = th.astype(np.float32)
+    _, _, g_all = s.eval(0, w)
+    s.close()
+    halves = []
+    for lo, hi in ((0, n // 2), (n // 2, n)):
+        mh = lib.default_model(n=hi - lo)
+        sh = lib.create(mh, lib.default_hmc(), lib.default_launch(), 1, 1)
+        sh.set_window_data(0, X[lo:hi], y[lo:hi])
+        halves.append(sh.eval(0, w)[2].astype(np.float64))
+        sh.close()
+    prior_g = w.astype(np.float64) * np.float32(-0.000025)
+    close_grad(halves[0] + halves[1] - prior_g, g_all.astype(np.float64), "additivity", rtol=3e-6)
+
+
+def test_residency_and_timeout_are_reported(pkg, lib):
+    m = lib.default_model(n=64)
+    with pytest.raises(pkg.BnnHmcError) as e:
+        lib.create(m, lib.default_hmc(), lib.default_launch(cus_per_chain=100000), 1, 1)
+    assert e.value.code == pkg.ERR_RESIDENCY
