@@ -1,0 +1,178 @@
+#!/usr/bin/env python3
+"""Benchmark of the HMC hot path on one MI355X.
+
+Workload (BASELINE.json configs[2]): independent windows of the 22->40->1 Bayesian MLP, full batch of
+58368 rows each (features ~ N(0,1), teacher-MLP targets + N(0, 0.01^2) noise, Gaussian likelihood,
+Gaussian weight prior), HMC with 1000 leapfrog steps per transition.  As many windows as are
+co-resident on the GPU form one batch; a "step" is one HMC transition (momentum resampling, 1000 fused
+leapfrog gradient evaluations, log accept ratio, Metropolis decision, adaptation, sample store) of
+every window of the batch.  The metric is leapfrog gradient evaluations per second; the minutes for
+200 windows x (100 burn-in + 800 samples) follow from it and are labelled as extrapolated unless
+--full runs that whole job.
+
+Prints ONE JSON line.  Inputs are resident in HBM before the timed region starts.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+N_ROWS, D0, D1 = 58368, 22, 40
+FLOP_PER_EVAL = 4 * N_ROWS * D1 * (D0 + 1)  # 214,794,240: both layers, forward + weight gradients
+PEAK_TFLOPS = 157.3                         # MI355X dense FP32 matrix peak (v_mfma_f32_16x16x4_f32)
+EVALS_200x800 = 200 * (900 * 1000 + 1)      # 200 windows x ((100 + 800) transitions x 1000 steps + bootstrap)
+EVALS_200x1600 = 200 * (1700 * 1000 + 1)
+
+
+def cpu_baseline(seconds):
+    """The CPU oracle (a port of the reference math), timed on this host's cores on one window."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import orc_binding as ob
+
+    orc = ob.load()
+    X, y, _ = orc.gen_window(0, 0, N_ROWS)
+    m = ob.gauss_model(n=N_ROWS)
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1)
+    threads = max(1, min(threads, os.cpu_count() or 1))
+    rate, used, done = orc.bench_grad_evals(m, X, y, threads, seconds)
+    return {"value": rate, "unit": "grad-evals/s", "cores": used, "kind": "port",
+            "sample": "%d leapfrog gradient evaluations of one 58368-row window in %.0f s, one chain per "
+                      "thread" % (done, seconds),
+            "extrapolated_minutes_200x800": EVALS_200x800 / rate / 60.0}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20, help="timed HMC transitions of the batch")
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--layer", choices=["mfma", "ffma"], default="mfma")
+    ap.add_argument("--cus-per-chain", type=int, default=0)
+    ap.add_argument("--wgs-per-cu", type=int, default=0)
+    ap.add_argument("--threads", type=int, default=0)
+    ap.add_argument("--pipeline", type=int, default=0)
+    ap.add_argument("--windows", type=int, default=0, help="0 = as many as are co-resident")
+    ap.add_argument("--leapfrog", type=int, default=1000)
+    ap.add_argument("--transitions-per-launch", type=int, default=5)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="0 skips the CPU baseline")
+    ap.add_argument("--full", action="store_true",
+                    help="run the whole 200 windows x (100 + 800) transitions job and time all of it")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU (windows are independent: more GPUs would only run more windows "
+              "side by side); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import __graft_entry__ as ge
+
+    pkg = ge.load_package()
+    lib = pkg.load()
+    rc, n_dev, cus, arch = lib.device_info()
+    if rc != 0:
+        print("no MI355X visible: %s" % lib.c.bnnhmc_last_error().decode(), file=sys.stderr)
+        sys.exit(1)
+
+    layer = pkg.LAYER_MFMA if args.layer == "mfma" else pkg.LAYER_FFMA
+    launch = lib.default_launch(layer=layer, transitions_per_launch=args.transitions_per_launch)
+    if args.cus_per_chain:
+        launch.cus_per_chain = args.cus_per_chain
+    if args.wgs_per_cu:
+        launch.wgs_per_cu = args.wgs_per_cu
+    if args.threads:
+        launch.threads = args.threads
+    if args.pipeline:
+        launch.pipeline = args.pipeline
+    wgs_per_cu = launch.wgs_per_cu if layer == pkg.LAYER_MFMA else 1
+    resident = max(1, (cus * wgs_per_cu) // launch.cus_per_chain)
+    n_windows = 200 if args.full else (args.windows or resident)
+
+    model = lib.default_model(lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
+    burn, keep = (100, 800) if args.full else (args.warmup + args.steps, 0)
+    hmc = lib.default_hmc(leapfrog_steps=args.leapfrog, burn_in=burn, n_samples=keep, seed=0)
+    s = lib.create(model, hmc, launch, n_windows, 1)
+    for w in range(n_windows):
+        s.generate_window(w, teacher_scale=0.1, noise_sigma=0.01)  # untimed, like the reference's load
+
+    if args.full:
+        # the reference's timed region: bootstrap + every transition (main.h:187-293)
+        t0 = time.perf_counter()
+        s.init_chains(None)
+        steps, warm, done = burn + keep, 0, 0
+        while done < steps:
+            k = min(25, steps - done)
+            s.run(k)
+            done += k
+            print("[bench] %d/%d transitions of %d windows, %.0f s" % (
+                done, steps, n_windows, time.perf_counter() - t0), file=sys.stderr, flush=True)
+        wall = time.perf_counter() - t0
+        tm0 = dict(kernel_ms=0.0, launches=0)
+    else:
+        s.init_chains(None)
+        steps, warm = args.steps, args.warmup
+        if warm:
+            s.run(warm)
+        tm0 = s.timing()
+        t0 = time.perf_counter()
+        s.run(steps)  # synchronous at return: the stream is drained
+        wall = time.perf_counter() - t0
+    tm1 = s.timing()
+    st = s.get_chain_state(0)
+    s.close()
+
+    evals = n_windows * steps * args.leapfrog + (n_windows if args.full else 0)
+    value = evals / wall
+    # dominant kernel: the trajectory kernel.  Average launch duration from HIP events recorded on the
+    # sampler's stream around the launches of the timed region.
+    dev_ms = tm1["kernel_ms"] - tm0["kernel_ms"]
+    launches = tm1["launches"] - tm0["launches"]
+    ms_per_launch = dev_ms / max(1, launches)
+    flop_per_launch = FLOP_PER_EVAL * (n_windows * steps * args.leapfrog) / max(1, launches)
+    achieved = flop_per_launch / (ms_per_launch * 1e-3) / 1e12
+
+    out = {
+        "metric": "leapfrog grad-evals/sec (minutes for 200 windows x 800 samples derived), 1 MI355X",
+        "value": value,
+        "unit": "grad-evals/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warm,
+        "ms_per_step": wall * 1e3 / steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[2]: %d independent windows x 1 chain (%d resident per launch), 22->40->1 BNN, "
+                        "58368x22 features ~N(0,1), teacher-MLP targets + N(0,0.01^2), Gaussian likelihood and "
+                        "prior, %d leapfrog steps per transition" % (n_windows, min(n_windows, resident),
+                                                                    args.leapfrog),
+            "layer": args.layer, "cus_per_chain": launch.cus_per_chain, "wgs_per_cu": wgs_per_cu,
+            "workgroups": tm1["workgroups"], "compute_units": cus,
+            "transitions_per_launch": args.transitions_per_launch,
+        },
+        "minutes_200x800": EVALS_200x800 / value / 60.0,
+        "minutes_200x800_kind": "measured: the whole job was run" if args.full
+                                else "extrapolated from the timed transitions",
+        "minutes_200x1600_extrapolated": EVALS_200x1600 / value / 60.0,
+        "reference_minutes_200x800_1xA100_tf32": 42,
+        "accept_rate_chain0": st["n_accepted"] / max(1, st["transitions_done"]),
+        "eps_chain0": st["eps"],
+        "roofline": {
+            "bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": achieved / PEAK_TFLOPS, "traffic": None,
+            "kernel": "hmc_kernel", "launches": launches, "ms_per_launch": ms_per_launch,
+            "flop_per_grad_eval": FLOP_PER_EVAL,
+        },
+    }
+    if args.cpu_seconds > 0:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -66,8 +66,12 @@ typedef struct bnnhmc_hmc {
 /* How the work is laid over the GPU.  Zero in a field selects the default. */
 typedef struct bnnhmc_launch {
   int layer;          /* BNNHMC_LAYER_MFMA (v_mfma_f32_16x16x4_f32) or BNNHMC_LAYER_FFMA          */
-  int cus_per_chain;  /* workgroups that share one chain's rows (default 32 = one XCD)           */
+  int cus_per_chain;  /* workgroups that share one chain's rows (default 8: 32 chains in flight)  */
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */
+  int threads;        /* threads per workgroup: 256, 512, 768 or 1024 (default 1024 for MFMA,    */
+                      /* 256 for FFMA)                                                           */
+  int pipeline;       /* MFMA layer: 1 = software-pipelined tile loop (512 threads), otherwise   */
+                      /* the plain tile loop (default)                                           */
   int transitions_per_launch; /* bound on one kernel's run time (default 8)                      */
   unsigned spin_limit; /* polls before an in-kernel wait gives up (default 1 << 22)              */
 } bnnhmc_launch;

@@ -34,6 +34,7 @@ class Hmc(C.Structure):
 
 class Launch(C.Structure):
     _fields_ = [("layer", C.c_int), ("cus_per_chain", C.c_int), ("wgs_per_cu", C.c_int),
+                ("threads", C.c_int), ("pipeline", C.c_int),
                 ("transitions_per_launch", C.c_int), ("spin_limit", C.c_uint)]
 
 

@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <string>
@@ -120,6 +121,8 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
     l.layer = lp->layer;
     if (lp->cus_per_chain > 0) l.cus_per_chain = lp->cus_per_chain;
     if (lp->wgs_per_cu > 0) l.wgs_per_cu = lp->wgs_per_cu;
+    if (lp->threads > 0) l.threads = lp->threads;
+    if (lp->pipeline > 0) l.pipeline = lp->pipeline;
     if (lp->transitions_per_launch > 0) l.transitions_per_launch = lp->transitions_per_launch;
     if (lp->spin_limit > 0) l.spin_limit = lp->spin_limit;
   }
@@ -127,9 +130,13 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
     return fail(BNNHMC_ERR_INVALID, "unknown layer variant %d", l.layer);
   if (l.wgs_per_cu < 1 || l.wgs_per_cu > 2)
     return fail(BNNHMC_ERR_INVALID, "wgs_per_cu must be 1 or 2, got %d", l.wgs_per_cu);
-  p.threads = (l.layer == BNNHMC_LAYER_MFMA && l.wgs_per_cu == 1) ? 512 : 256;
-  p.kernel = hmc_kernel_for(m.d0, m.d1, l.layer, m.lik_kind, p.threads);
-  if (!p.kernel) return fail(BNNHMC_ERR_INVALID, "no kernel for this configuration");
+  const bool piped = l.layer == BNNHMC_LAYER_MFMA && l.pipeline == 1;
+  p.threads = l.threads > 0 ? l.threads
+                            : (l.layer == BNNHMC_LAYER_FFMA || l.wgs_per_cu == 2 ? 256 : (piped ? 512 : 1024));
+  p.kernel = hmc_kernel_for(m.d0, m.d1, l.layer, m.lik_kind, p.threads, piped ? 1 : 0);
+  if (!p.kernel)
+    return fail(BNNHMC_ERR_INVALID, "no kernel for layer %d with %d threads per workgroup", l.layer,
+                p.threads);
   int per_cu = 0;
   HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, p.kernel, p.threads, 0));
   if (per_cu < 1) return fail(BNNHMC_ERR_RESIDENCY, "kernel does not fit a compute unit");
@@ -242,6 +249,7 @@ struct bnnhmc_sampler {
   float* tmp = nullptr;       // evaluation scratch: w | grad | prior (3 * st_stride) ...
   float* tmp_ell = nullptr;   // ... and n_pad rows
   double* tmp_sums = nullptr; // [max_groups][2]
+  unsigned long long* debug_phase = nullptr;  // set when BNNHMC_DEBUG_PHASE is in the environment
   // timing
   double kernel_ms = 0.0;
   long launches = 0, grad_evals = 0;
@@ -364,8 +372,10 @@ void bnnhmc_default_hmc(bnnhmc_hmc* h) {
 void bnnhmc_default_launch(bnnhmc_launch* l) {
   if (!l) return;
   l->layer = BNNHMC_LAYER_MFMA;
-  l->cus_per_chain = 32;
+  l->cus_per_chain = 8;
   l->wgs_per_cu = 1;
+  l->threads = 0;
+  l->pipeline = 0;
   l->transitions_per_launch = 8;
   l->spin_limit = 1u << 22;
 }
@@ -610,6 +620,9 @@ int bnnhmc_create(const bnnhmc_model* model, const bnnhmc_hmc* hmc, const bnnhmc
       (rc = s->alloc(&s->tmp_sums, (size_t)2 * eval_groups_max)))
     return bail(rc);
   s->workspace = ws;
+  if (getenv("BNNHMC_DEBUG_PHASE")) {
+    if ((rc = s->alloc(&s->debug_phase, (size_t)8 * 4096))) return bail(rc);
+  }
   e = hipMemsetAsync(s->y, 0, (size_t)n_windows * s->n_pad * sizeof(float), s->stream);
   if (e == hipSuccess) e = hipMemsetAsync(ws, 0, s->workspace_bytes, s->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(s->stream);
@@ -750,6 +763,7 @@ int bnnhmc_run(bnnhmc_sampler* s, int n_transitions) {
       a.tr_eps = s->tr_eps;
       a.trace_len = s->trace_len;
       a.seed = s->hmc.seed;
+      a.debug_phase = s->debug_phase;
       int rc = launch_and_count(s, a, groups);
       if (rc) return rc;
       ++launches;
@@ -760,6 +774,20 @@ int bnnhmc_run(bnnhmc_sampler* s, int n_transitions) {
   if (rc) return rc;
   float ms = 0.0f;
   HIP_TRY(hipEventElapsedTime(&ms, s->ev0, s->ev1));
+  if (s->debug_phase) {
+    // cycles per phase of the last launch, averaged over its workgroups
+    std::vector<unsigned long long> h((size_t)8 * s->last_workgroups);
+    HIP_TRY(hipMemcpy(h.data(), s->debug_phase, h.size() * sizeof(h[0]), hipMemcpyDeviceToHost));
+    double tot[8] = {0};
+    for (int wgi = 0; wgi < s->last_workgroups; ++wgi)
+      for (int k = 0; k < 8; ++k) tot[k] += (double)h[(size_t)wgi * 8 + k] / s->last_workgroups;
+    const char* names[8] = {"update+sync", "operand fetch", "tile loop", "partials->LDS+sync",
+                            "stage1+store", "group barrier", "stage2", "epilogue"};
+    double sum = 0;
+    for (int k = 0; k < 8; ++k) sum += tot[k];
+    for (int k = 0; k < 8; ++k)
+      fprintf(stderr, "[bnnhmc phase] %-20s %14.0f ticks %6.2f%%\n", names[k], tot[k], 100.0 * tot[k] / sum);
+  }
   s->kernel_ms += ms;
   s->launches += launches;
   s->grad_evals += (long)s->n_chains * n_transitions * s->hmc.leapfrog_steps;

@@ -112,6 +112,7 @@ struct KArgs {
   unsigned* status;    // [0] abort flag, [1] timed-out workgroup + 1
   unsigned spin_limit;
   unsigned* debug_xcc; // optional [workgroup] XCC id
+  unsigned long long* debug_phase;  // optional [workgroup][8] cycles spent per phase of a step
 };
 
 }  // namespace bnn

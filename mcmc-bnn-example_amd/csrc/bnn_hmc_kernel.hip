@@ -113,6 +113,27 @@ struct StepCtx {
   float* ell_new;         // last step only: where to store this state's rows (null = skip)
 };
 
+// Constant operand slots of the MFMA layer: `one` reads (1, 0) at offsets j * D0 (j < 4), `zero` reads
+// (0, 0); lanes holding the appended constant-one feature or tile padding point here.
+template <int D0>
+struct AugTable {
+  float one[3 * D0 + 4];
+  float zero[3 * D0 + 4];
+};
+template <int D0>
+constexpr AugTable<D0> make_aug_table() {
+  AugTable<D0> t{};
+  for (int j = 0; j < 4; ++j) t.one[j * D0] = 1.0f;
+  return t;
+}
+__device__ const AugTable<22> k_aug_table_22 = make_aug_table<22>();
+template <int D0>
+__device__ __forceinline__ const AugTable<D0>* aug_table();
+template <>
+__device__ __forceinline__ const AugTable<22>* aug_table<22>() {
+  return &k_aug_table_22;
+}
+
 // ================================================================================================
 // MFMA layer: both contractions on v_mfma_f32_16x16x4_f32.
 //
@@ -128,7 +149,7 @@ struct StepCtx {
 // GEMM2; the contraction index of GEMM1 and the feature index of GEMM2 are permuted so that every
 // lane reads contiguous floats of a row.
 // ================================================================================================
-template <int D0, int D1>
+template <int D0, int D1, int PIPE>
 struct MfmaLayer {
   static_assert(D0 % 2 == 0, "feature pairs are read as float2");
   static constexpr int KS = (D0 + 1 + 3) / 4;  // k-steps of GEMM1 (one more feature: the bias)
@@ -139,12 +160,12 @@ struct MfmaLayer {
   static constexpr int oB1 = D0 * D1, oW2 = oB1 + D1, oB2 = oW2 + D1, P = oB2 + 1;
   static constexpr int P_AL = (P + 3) / 4 * 4;
 
-  float w1b[KS][NT];
-  float w2v[NT];
-  float b2;
+  float w1b[KS][NT];   // W1_aug scaled by -2/ln 2: GEMM1 yields the exp2 argument of the activation
+  float w2v[NT];       // w2[c]
+  float w2y[NT];       // -w2[c] / lik_scale: the layer-2 dot yields the scaled residual directly
+  float yh_init;       // -b2 / lik_scale in lane n == 0, else 0
   f4 dacc[NT][2];
   float dw2acc[NT];
-  float db2acc;
   double dl;
 
   struct TileIn {
@@ -153,7 +174,9 @@ struct MfmaLayer {
     f4 yv;
   };
 
-  __device__ __forceinline__ void load_weights(const float* s_w) {
+  static constexpr float kExp2Scale = -2.88539008177792681472f;  // -2 / ln 2, kernel_helpers.h:37
+
+  __device__ __forceinline__ void load_weights(const float* s_w, const ModelConsts& mc) {
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -166,11 +189,12 @@ struct MfmaLayer {
         float v = 0.0f;
         if (k < D0) v = s_w[k * D1 + cc];
         else if (k == D0) v = s_w[oB1 + cc];
-        w1b[s][t] = cv ? v : 0.0f;
+        w1b[s][t] = cv ? v * kExp2Scale : 0.0f;
       }
       w2v[t] = cv ? s_w[oW2 + cc] : 0.0f;
+      w2y[t] = -w2v[t] * mc.scale_recp;
     }
-    b2 = s_w[oB2];
+    yh_init = n == 0 ? -s_w[oB2] * mc.scale_recp : 0.0f;
   }
 
   __device__ __forceinline__ void zero_acc() {
@@ -180,34 +204,10 @@ struct MfmaLayer {
       dacc[t][1] = f4{0.f, 0.f, 0.f, 0.f};
       dw2acc[t] = 0.0f;
     }
-    db2acc = 0.0f;
     dl = 0.0;
   }
 
-  __device__ __forceinline__ void load_tile_fast(TileIn& ti, const StepCtx& cx, int row0, int n,
-                                                 int q) const {
-    const float* ra = cx.X + (size_t)(row0 + n) * D0;
-#pragma unroll
-    for (int i = 0; i < KP; ++i) {
-      const int k0 = KS * q + 2 * i;
-      const int kc = k0 < D0 ? k0 : D0 - 2;
-      f2 v = *reinterpret_cast<const f2*>(ra + kc);
-      if (k0 >= D0) v = f2{k0 == D0 ? 1.0f : 0.0f, 0.0f};
-      ti.xa[i] = v;
-    }
-    const int f0 = 2 * n;
-    const int fc = f0 < D0 ? f0 : D0 - 2;
-    const float* rb = cx.X + (size_t)(row0 + 4 * q) * D0 + fc;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      f2 v = *reinterpret_cast<const f2*>(rb + j * D0);
-      if (f0 >= D0) v = f2{f0 == D0 ? 1.0f : 0.0f, 0.0f};
-      ti.xb[j] = v;
-    }
-    ti.yv = *reinterpret_cast<const f4*>(cx.y + row0 + 4 * q);
-  }
-
-  // any alignment, rows past the end read as the last row (their gradient is masked to zero)
+  // rows past the end read as the last row (their gradient is masked to zero); any alignment
   __device__ __forceinline__ void load_tile_safe(TileIn& ti, const StepCtx& cx, int row0, int n,
                                                  int q) const {
     const int last = cx.n - 1;
@@ -234,52 +234,54 @@ struct MfmaLayer {
     }
   }
 
-  __device__ __forceinline__ void load_tile(TileIn& ti, const StepCtx& cx, int tile, int n,
-                                            int q) const {
-    const int row0 = tile * 16;
-    if (cx.x_vec_ok && cx.y_vec_ok && row0 + 16 <= cx.n) load_tile_fast(ti, cx, row0, n, q);
-    else load_tile_safe(ti, cx, row0, n, q);
-  }
-
-  template <int LIK, bool LAST>
-  __device__ __forceinline__ void compute_tile(const TileIn& ti, const StepCtx& cx,
-                                               const ModelConsts& mc, int row0, int n, int q) {
-    // ---- GEMM1: pre-activations (bias included through the constant-one feature) ----
-    f4 acc[NT];
+  // ---- the four stages of a tile ----
+  // B: GEMM1, pre-activations (bias included through the constant-one feature)
+  __device__ __forceinline__ void gemm1(const f2 (&xa)[KP], f4 (&acc)[NT]) const {
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < KP; ++i) {
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(ti.xa[i][0], w1b[2 * i][t], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[i][0], w1b[2 * i][t], acc[t], 0, 0, 0);
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        acc[t] =
-            __builtin_amdgcn_mfma_f32_16x16x4f32(ti.xa[i][1], w1b[2 * i + 1][t], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[i][1], w1b[2 * i + 1][t], acc[t], 0, 0, 0);
     }
-    // ---- activation, layer-2 dot ----
-    float yh[4] = {0.f, 0.f, 0.f, 0.f};
+  }
+
+  // C: activation, layer-2 dot, per-row loss gradient, layer-2 weight gradient, delta (in place).
+  // acc arrives as the exp2 argument t = -2 x / ln 2 of tanh(x) = 2 / (1 + 2^t) - 1
+  // (kernel_helpers.h:34-42 without its small-|x| identity branch, which changes the value by less
+  // than 1.5e-7).  delta leaves without the factor w2[c], which is applied once per step to the
+  // GEMM2 result; the padded hidden units (zero weights: h = 0) then carry delta = g, so the
+  // constant-one column of GEMM2 delivers db2 in row c = D1 for free.
+  template <int LIK, bool LAST, bool FULL>
+  __device__ __forceinline__ void pointwise(f4 (&acc)[NT], const f4& yv, const StepCtx& cx,
+                                            const ModelConsts& mc, int row0, int n, int q) {
+    float yh[4] = {yh_init, yh_init, yh_init, yh_init};
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        acc[t][j] = tanh_fwd(acc[t][j]);
-        yh[j] = __builtin_fmaf(w2v[t], acc[t][j], yh[j]);
+        const float e = __builtin_amdgcn_exp2f(acc[t][j]);
+        const float sg = __builtin_amdgcn_rcpf(1.0f + e);
+        const float h = __builtin_fmaf(sg, 2.0f, -1.0f);
+        acc[t][j] = h;
+        yh[j] = __builtin_fmaf(w2y[t], h, yh[j]);
       }
     }
-    // ---- per-row loss gradient ----
     float g[4];
-    float gsum = 0.0f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float yhat = row16_allreduce(yh[j]);
-      float diff;
-      float gj = lik_grad<LIK>(mc, ti.yv[j] - yhat - b2, diff);
-      const bool valid = row0 + 4 * q + j < cx.n;
+      // scaled residual (y - yhat - b2) / scale, mcmc_step_ffma.h:293
+      const float diff = __builtin_fmaf(yv[j], mc.scale_recp, row16_allreduce(yh[j]));
+      float gj;
+      if (LIK == 0) gj = diff * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(diff, diff, mc.df));
+      else gj = diff * mc.scale_recp;
+      const bool valid = FULL || (row0 + 4 * q + j < cx.n);
       gj = valid ? gj : 0.0f;  // mcmc_step_ffma.h:301
       g[j] = gj;
-      gsum += gj;
       if (LAST) {
         if (n == 0 && valid) {
           const int row = row0 + 4 * q + j;
@@ -290,45 +292,161 @@ struct MfmaLayer {
         }
       }
     }
-    db2acc += gsum;
-    // ---- layer-2 weight gradient, delta = (1 - h^2) w2 g ----
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float h = acc[t][j];
         dw2acc[t] = __builtin_fmaf(g[j], h, dw2acc[t]);
-        acc[t][j] = __builtin_fmaf(-h, h, 1.0f) * (w2v[t] * g[j]);
+        acc[t][j] = __builtin_fmaf(-h, h, 1.0f) * g[j];
       }
     }
-    // ---- GEMM2: dW1_aug^T += delta^T X_aug ----
+  }
+
+  // D: GEMM2, dW1_aug^T += delta^T X_aug
+  __device__ __forceinline__ void gemm2(const f4 (&dlt)[NT], const f2 (&xb)[4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        dacc[t][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(acc[t][j], ti.xb[j][0], dacc[t][0], 0, 0, 0);
-        dacc[t][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(acc[t][j], ti.xb[j][1], dacc[t][1], 0, 0, 0);
+        dacc[t][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(dlt[t][j], xb[j][0], dacc[t][0], 0, 0, 0);
+        dacc[t][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(dlt[t][j], xb[j][1], dacc[t][1], 0, 0, 0);
       }
+    }
+  }
+
+  // Software-pipelined loop over full, aligned tiles [tb, te).  Iteration i issues the loads of tile
+  // i + 2, GEMM1 of tile i + 1, the pointwise work of tile i and GEMM2 of tile i - 1, all in one
+  // basic block, so the matrix pipe (42 MFMAs per tile) and the vector ALU (the pointwise work) run
+  // side by side inside one wave.  Lanes whose operand slot is the constant-one feature or padding
+  // read it from a small constant table through a per-lane pointer with stride zero, so no select
+  // sits between a load and its use.
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void fast_loop(const StepCtx& cx, const ModelConsts& mc, int tb, int te,
+                                            int n, int q) {
+    const AugTable<D0>* aug = aug_table<D0>();
+    const size_t tile_floats = (size_t)16 * D0;
+    // A operand: pairs 0 .. KP-2 are always real features; the last pair of lane group q = 3 is
+    // the (1, 0) constant
+    const float* pa = cx.X + (size_t)n * D0 + KS * q;
+    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
+    const float* pa_last0 = a_const ? aug->one : pa + (size_t)tb * tile_floats + 2 * (KP - 1);
+    const unsigned sa_last = a_const ? 0u : (unsigned)tile_floats;
+    // B operand of GEMM2: feature pair 2n, 2n+1 of rows 4q + j
+    const bool b_const = 2 * n >= D0;
+    const float* pb0 = b_const ? (2 * n == D0 ? aug->one : aug->zero)
+                               : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 2 * n;
+    const unsigned sb = b_const ? 0u : (unsigned)tile_floats;
+    const float* py = cx.y + 4 * q;
+
+    auto load = [&](TileIn& ti, int tile) {
+      const float* ra = pa + (size_t)tile * tile_floats;
+#pragma unroll
+      for (int i = 0; i < KP - 1; ++i) ti.xa[i] = *reinterpret_cast<const f2*>(ra + 2 * i);
+      const unsigned rel = (unsigned)(tile - tb);
+      ti.xa[KP - 1] = *reinterpret_cast<const f2*>(pa_last0 + (size_t)rel * sa_last);
+      const float* rb = pb0 + (size_t)rel * sb;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ti.xb[j] = *reinterpret_cast<const f2*>(rb + j * D0);
+      ti.yv = *reinterpret_cast<const f4*>(py + (size_t)tile * 16);
+    };
+
+    TileIn t0, t1, t2;  // tiles i, i + 1, i + 2
+    f4 acc_cur[NT], acc_nxt[NT], dlt_prev[NT];
+    f2 xb_prev[4];
+    load(t0, tb);
+    load(t1, tb + 1 < te ? tb + 1 : tb);
+    gemm1(t0.xa, acc_cur);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) dlt_prev[t] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xb_prev[j] = t0.xb[j];
+    for (int i = tb; i < te; ++i) {
+      load(t2, i + 2 < te ? i + 2 : te - 1);
+      gemm1(t1.xa, acc_nxt);                                       // tile i + 1
+      gemm2(dlt_prev, xb_prev);                                    // tile i - 1 (zero delta at i = tb)
+      pointwise<LIK, LAST, true>(acc_cur, t0.yv, cx, mc, i * 16, n, q);  // tile i -> delta in acc_cur
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        dlt_prev[t] = acc_cur[t];
+        acc_cur[t] = acc_nxt[t];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xb_prev[j] = t0.xb[j];
+      t0 = t1;
+      t1 = t2;
+    }
+    gemm2(dlt_prev, xb_prev);  // tile te - 1
+  }
+
+  // Plain loop over full, aligned tiles [tb, te): loads one tile ahead, then GEMM1, pointwise work
+  // and GEMM2 of the current tile back to back.  Needs few registers, so more waves fit a SIMD and
+  // fill each other's dependency and memory stalls.
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void simple_loop(const StepCtx& cx, const ModelConsts& mc, int tb,
+                                              int te, int n, int q) {
+    const AugTable<D0>* aug = aug_table<D0>();
+    const size_t tile_floats = (size_t)16 * D0;
+    const float* pa = cx.X + (size_t)n * D0 + KS * q;
+    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
+    const float* pa_last0 = a_const ? aug->one : pa + (size_t)tb * tile_floats + 2 * (KP - 1);
+    const unsigned sa_last = a_const ? 0u : (unsigned)tile_floats;
+    const bool b_const = 2 * n >= D0;
+    const float* pb0 = b_const ? (2 * n == D0 ? aug->one : aug->zero)
+                               : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 2 * n;
+    const unsigned sb = b_const ? 0u : (unsigned)tile_floats;
+    const float* py = cx.y + 4 * q;
+    auto load = [&](TileIn& ti, int tile) {
+      const float* ra = pa + (size_t)tile * tile_floats;
+#pragma unroll
+      for (int i = 0; i < KP - 1; ++i) ti.xa[i] = *reinterpret_cast<const f2*>(ra + 2 * i);
+      const unsigned rel = (unsigned)(tile - tb);
+      ti.xa[KP - 1] = *reinterpret_cast<const f2*>(pa_last0 + (size_t)rel * sa_last);
+      const float* rb = pb0 + (size_t)rel * sb;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ti.xb[j] = *reinterpret_cast<const f2*>(rb + j * D0);
+      ti.yv = *reinterpret_cast<const f4*>(py + (size_t)tile * 16);
+    };
+    TileIn cur, nx1, nx2;  // loads run two tiles ahead of their use
+    load(cur, tb);
+    load(nx1, tb + 1 < te ? tb + 1 : te - 1);
+    for (int i = tb; i < te; ++i) {
+      load(nx2, i + 2 < te ? i + 2 : te - 1);
+      f4 acc[NT];
+      gemm1(cur.xa, acc);
+      pointwise<LIK, LAST, true>(acc, cur.yv, cx, mc, i * 16, n, q);
+      gemm2(acc, cur.xb);
+      cur = nx1;
+      nx1 = nx2;
     }
   }
 
   template <int LIK, bool LAST>
   __device__ __forceinline__ void run_tiles(const StepCtx& cx, const ModelConsts& mc) {
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
-    if (cx.tile_begin >= cx.tile_end) return;
-    TileIn cur, nxt;
-    load_tile(cur, cx, cx.tile_begin, n, q);
-    for (int tile = cx.tile_begin; tile < cx.tile_end; ++tile) {
-      const int tn = tile + 1 < cx.tile_end ? tile + 1 : tile;
-      load_tile(nxt, cx, tn, n, q);  // prefetch
-      compute_tile<LIK, LAST>(cur, cx, mc, tile * 16, n, q);
-      cur = nxt;
+    const int tb = cx.tile_begin, te = cx.tile_end;
+    int fast_end = tb;
+    if (cx.x_vec_ok && cx.y_vec_ok) fast_end = min(te, cx.n / 16);
+    if (fast_end > tb) {
+      if (PIPE) fast_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
+      else simple_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
+    }
+    // ragged tail tile, or unaligned caller buffers: one tile at a time
+    for (int tile = max(tb, fast_end); tile < te; ++tile) {
+      TileIn ti;
+      f4 acc[NT];
+      load_tile_safe(ti, cx, tile * 16, n, q);
+      gemm1(ti.xa, acc);
+      pointwise<LIK, LAST, false>(acc, ti.yv, cx, mc, tile * 16, n, q);
+      gemm2(acc, ti.xb);
     }
   }
 
-  // this wave's partial sums -> its LDS slot, indexed by canonical parameter number
-  __device__ __forceinline__ void write_partials(float* slot) {
+  // this wave's partial sums -> its LDS slot, indexed by canonical parameter number; the factor
+  // w2[c] left out of delta is applied here
+  __device__ __forceinline__ void write_partials(float* slot, const float* s_w) {
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    static_assert(D1 % 16 != 0, "db2 rides in the first padded hidden unit");
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -338,8 +456,11 @@ struct MfmaLayer {
         for (int j = 0; j < 4; ++j) {
           const int c = 16 * t + 4 * q + j;
           if (c < D1) {
-            if (f < D0) slot[f * D1 + c] = dacc[t][u][j];
-            else if (f == D0) slot[oB1 + c] = dacc[t][u][j];
+            const float v = dacc[t][u][j] * s_w[oW2 + c];
+            if (f < D0) slot[f * D1 + c] = v;
+            else if (f == D0) slot[oB1 + c] = v;
+          } else if (c == D1 && f == D0) {
+            slot[oB2] = dacc[t][u][j];  // sum of g over this wave's rows
           }
         }
       }
@@ -350,14 +471,10 @@ struct MfmaLayer {
       const int c = 16 * t + n;
       if (q == 0 && c < D1) slot[oW2 + c] = v;
     }
-    float b = db2acc;
-    b += __shfl_xor(b, 16);
-    b += __shfl_xor(b, 32);
     double d = dl;  // held by lanes n == 0
     d += shfl_xor_d(d, 16);
     d += shfl_xor_d(d, 32);
     if (lane == 0) {
-      slot[oB2] = b;
       const uint64_t bits = double_to_bits(d);
       slot[P_AL] = __builtin_bit_cast(float, (uint32_t)bits);
       slot[P_AL + 1] = __builtin_bit_cast(float, (uint32_t)(bits >> 32));
@@ -396,7 +513,7 @@ struct FfmaLayer {
     float yv;
   };
 
-  __device__ __forceinline__ void load_weights(const float* s_w) {
+  __device__ __forceinline__ void load_weights(const float* s_w, const ModelConsts&) {
     const int lane = threadIdx.x & 63, cc = lane & 7;
 #pragma unroll
     for (int i = 0; i < HU; ++i) {
@@ -507,7 +624,7 @@ struct FfmaLayer {
     return v;
   }
 
-  __device__ __forceinline__ void write_partials(float* slot) {
+  __device__ __forceinline__ void write_partials(float* slot, const float*) {
     const int lane = threadIdx.x & 63, cc = lane & 7, rg = lane >> 3;
 #pragma unroll
     for (int i = 0; i < HU; ++i) {
@@ -604,7 +721,8 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   if (group >= a.n_groups) return;
   const int chain = a.chain_base + group;
   const int window = a.fixed_window >= 0 ? a.fixed_window : chain / a.chains_per_window;
-  const int tid = threadIdx.x, wave = tid >> 6;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
 
   StepCtx cx;
   cx.X = a.X + (size_t)window * a.x_stride;
@@ -658,6 +776,17 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
 
   Layer layer;
   bool ok = true;
+  // optional per-phase cycle accounting (thread 0 of each workgroup)
+  unsigned long long ph[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  unsigned long long tstamp = 0;
+  const bool prof = a.debug_phase != nullptr;
+#define BNN_PHASE(k)                                        \
+  if (prof) {                                               \
+    const unsigned long long now_ = __builtin_readcyclecounter(); \
+    ph[k] += now_ - tstamp;                                 \
+    tstamp = now_;                                          \
+  }
+  if (prof) tstamp = __builtin_readcyclecounter();
   const int n_outer = trans ? a.n_trans : 1;
   double dl_total = 0.0;
 
@@ -696,8 +825,10 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         }
       }
       __syncthreads();
-      layer.load_weights(s_w);
+      BNN_PHASE(0)  // update + sync
+      layer.load_weights(s_w, mc);
       layer.zero_acc();
+      BNN_PHASE(1)  // operand fetch from LDS
       const bool last = s == a.L - 1;
       if (last) {
         cx.ell_prev = ell_cur;
@@ -706,8 +837,10 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       } else {
         layer.template run_tiles<LIK, false>(cx, mc);
       }
-      layer.write_partials(s_slots[wave]);
+      BNN_PHASE(2)  // tile loop
+      layer.write_partials(s_slots[wave], s_w);
       __syncthreads();
+      BNN_PHASE(3)  // wave partials -> LDS + sync
       // ---- stage 1: fixed-order sum over this workgroup's waves -> global partial record ----
       float* my_part = part_base + ((size_t)buf * a.G + rank) * SLOT;
 #pragma unroll
@@ -732,9 +865,11 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         st_agent(my_part + P_AL, __builtin_bit_cast(float, (uint32_t)bits));
         st_agent(my_part + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)));
       }
+      BNN_PHASE(4)  // stage 1 + global store
       bar_target += (unsigned)a.G;
       ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag);
       if (!ok) break;
+      BNN_PHASE(5)  // group barrier
       // ---- stage 2: fixed-order sum over the group's workgroups; the prior gradient seeds the sum
       //      as block 0 does in the reference (mcmc_step_ffma.h:144) ----
       const float* grp_part = part_base + (size_t)buf * a.G * SLOT;
@@ -743,7 +878,17 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         const int p = tid + i * T;
         if (p < P) {
           float v = prior_grad(mc, w[i]);
-          for (int r = 0; r < a.G; ++r) v += ld_agent(grp_part + (size_t)r * SLOT + p);
+          // eight loads in flight at a time; the additions keep the order r = 0, 1, 2, ...
+          for (int r0 = 0; r0 < a.G; r0 += 8) {
+            float t8[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+              const int r = r0 + k < a.G ? r0 + k : a.G - 1;
+              t8[k] = ld_agent(grp_part + (size_t)r * SLOT + p);
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v += r0 + k < a.G ? t8[k] : 0.0f;
+          }
           g[i] = v;
         }
       }
@@ -758,6 +903,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         dl_total = d;
       }
       buf ^= 1;
+      BNN_PHASE(6)  // stage 2
     }
     if (!ok) break;
 
@@ -823,6 +969,12 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
     }
   }
 
+  if (prof && tid == 0) {
+    BNN_PHASE(7)  // transition epilogue
+#pragma unroll
+    for (int k = 0; k < 8; ++k) a.debug_phase[(size_t)blockIdx.x * 8 + k] = ph[k];
+  }
+#undef BNN_PHASE
   if (!ok) return;
   // ---- write back ----
   if (rank == 0) {
@@ -883,13 +1035,19 @@ static const void* kernel_ptr() {
   return reinterpret_cast<const void*>(&hmc_kernel<Layer, LIK, T>);
 }
 
-const void* hmc_kernel_for(int d0, int d1, int layer, int lik, int threads) {
+const void* hmc_kernel_for(int d0, int d1, int layer, int lik, int threads, int pipeline) {
   if (d0 != 22 || d1 != 40) return nullptr;
-  using M = MfmaLayer<22, 40>;
+  using MP = MfmaLayer<22, 40, 1>;
+  using MS = MfmaLayer<22, 40, 0>;
   using F = FfmaLayer<22, 40>;
-  if (layer == 0) {
-    if (threads == 512) return lik == 0 ? kernel_ptr<M, 0, 512>() : kernel_ptr<M, 1, 512>();
-    if (threads == 256) return lik == 0 ? kernel_ptr<M, 0, 256>() : kernel_ptr<M, 1, 256>();
+  if (layer == 0 && pipeline) {
+    if (threads == 512) return lik == 0 ? kernel_ptr<MP, 0, 512>() : kernel_ptr<MP, 1, 512>();
+    if (threads == 256) return lik == 0 ? kernel_ptr<MP, 0, 256>() : kernel_ptr<MP, 1, 256>();
+  } else if (layer == 0) {
+    if (threads == 1024) return lik == 0 ? kernel_ptr<MS, 0, 1024>() : kernel_ptr<MS, 1, 1024>();
+    if (threads == 768) return lik == 0 ? kernel_ptr<MS, 0, 768>() : kernel_ptr<MS, 1, 768>();
+    if (threads == 512) return lik == 0 ? kernel_ptr<MS, 0, 512>() : kernel_ptr<MS, 1, 512>();
+    if (threads == 256) return lik == 0 ? kernel_ptr<MS, 0, 256>() : kernel_ptr<MS, 1, 256>();
   } else if (layer == 1) {
     if (threads == 256) return lik == 0 ? kernel_ptr<F, 0, 256>() : kernel_ptr<F, 1, 256>();
   }

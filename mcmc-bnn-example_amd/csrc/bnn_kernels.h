@@ -8,8 +8,9 @@
 
 namespace bnn {
 
-// trajectory kernel for (d0, d1, layer, likelihood, threads per workgroup); nullptr if unsupported
-const void* hmc_kernel_for(int d0, int d1, int layer, int lik, int threads);
+// trajectory kernel for (d0, d1, layer, likelihood, threads per workgroup, software-pipelined tile
+// loop or plain loop); nullptr if unsupported
+const void* hmc_kernel_for(int d0, int d1, int layer, int lik, int threads, int pipeline);
 hipError_t launch_hmc_kernel(const void* kernel, const KArgs& args, int workgroups, int threads,
                              hipStream_t stream);
 
