@@ -26,6 +26,10 @@ FLOP_PER_EVAL = 4 * N_ROWS * D1 * (D0 + 1)  # 214,794,240: both layers, forward 
 PEAK_TFLOPS = 157.3                         # MI355X dense FP32 matrix peak (v_mfma_f32_16x16x4_f32)
 EVALS_200x800 = 200 * (900 * 1000 + 1)      # 200 windows x ((100 + 800) transitions x 1000 steps + bootstrap)
 EVALS_200x1600 = 200 * (1700 * 1000 + 1)
+# HBM-side bytes per gradient evaluation of the MFMA trajectory kernel, from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE scaled by a 1 GiB copy kernel (profiles/hmc_kernel_mfma_22x40_32windows.txt): one window's
+# X and y (5.37 MB) pass through L2 once per leapfrog step, plus the partial-gradient records.
+TRAFFIC_BYTES_PER_EVAL_MFMA = 9.388e11 / 160000
 
 
 def cpu_baseline(seconds):
@@ -49,7 +53,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20, help="timed HMC transitions of the batch")
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layer", choices=["mfma", "ffma"], default="mfma")
     ap.add_argument("--cus-per-chain", type=int, default=0)
     ap.add_argument("--wgs-per-cu", type=int, default=0)
@@ -164,7 +168,10 @@ def main():
         "eps_chain0": st["eps"],
         "roofline": {
             "bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": achieved / PEAK_TFLOPS, "traffic": None,
+            "frac": achieved / PEAK_TFLOPS,
+            "traffic": (TRAFFIC_BYTES_PER_EVAL_MFMA * n_windows * steps * args.leapfrog / max(1, launches)
+                        if args.layer == "mfma" else None),
+            "traffic_unit": "bytes per launch (measured offline with rocprofv3 --pmc, see profiles/)",
             "kernel": "hmc_kernel", "launches": launches, "ms_per_launch": ms_per_launch,
             "flop_per_grad_eval": FLOP_PER_EVAL,
         },

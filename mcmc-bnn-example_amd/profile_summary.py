@@ -1,0 +1,86 @@
+#!/usr/bin/env python3
+"""Condenses the raw rocprofv3 output written by profile.sh into a few lines of text."""
+import collections
+import csv
+import glob
+import json
+import os
+import sys
+
+
+def find(d, pat):
+    hits = glob.glob(os.path.join(d, "**", pat), recursive=True)
+    return hits[0] if hits else None
+
+
+def counter_totals(path, kernel_substr):
+    """{dispatch: {counter: sum over instances}} for kernels whose name contains kernel_substr"""
+    agg = collections.defaultdict(lambda: collections.defaultdict(float))
+    for r in csv.DictReader(open(path)):
+        if kernel_substr in r["Kernel_Name"]:
+            agg[r["Dispatch_Id"]][r["Counter_Name"]] += float(r["Counter_Value"])
+    return agg
+
+
+def main(out):
+    lines = []
+    stats = find(os.path.join(out, "trace"), "*kernel_stats.csv")
+    if stats:
+        lines.append("kernel stats (rocprofv3 --kernel-trace --stats):")
+        lines.append("  %-70s %8s %14s %14s %7s" % ("kernel", "calls", "total ms", "avg ms", "%"))
+        for r in csv.DictReader(open(stats)):
+            lines.append("  %-70s %8s %14.3f %14.3f %7.2f" % (
+                r["Name"][:70], r["Calls"], float(r["TotalDurationNs"]) / 1e6,
+                float(r["AverageNs"]) / 1e6, float(r["Percentage"])))
+    kt = find(os.path.join(out, "trace"), "*kernel_trace.csv")
+    if kt:
+        durs = [(int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e6
+                for r in csv.DictReader(open(kt)) if "hmc_kernel" in r["Kernel_Name"]]
+        lines.append("hmc_kernel dispatch durations, ms (the first is the bootstrap evaluation, then one per "
+                     "launch of transitions): " + ", ".join("%.3f" % d for d in durs))
+        big = [d for d in durs if d > 0.5 * max(durs)]
+        if big:
+            lines.append("average over the %d full-size launches: %.3f ms" % (len(big), sum(big) / len(big)))
+    bj = os.path.join(out, "bench_trace.json")
+    if os.path.exists(bj):
+        try:
+            d = json.loads(open(bj).read().strip().splitlines()[-1])
+            lines.append("bench.py under the tracer: %.0f grad-evals/s, roofline frac %.3f, %.3f ms per launch "
+                         "(HIP events), %d launches" % (d["value"], d["roofline"]["frac"],
+                                                        d["roofline"]["ms_per_launch"], d["roofline"]["launches"]))
+        except Exception as e:  # noqa: BLE001
+            lines.append("bench json unreadable: %r" % e)
+    scale = {}
+    for c in ("FETCH_SIZE", "WRITE_SIZE"):
+        cp = find(os.path.join(out, "copy_" + c), "*counter_collection.csv")
+        kp = find(os.path.join(out, "pmc_" + c), "*counter_collection.csv")
+        if cp:
+            tot = counter_totals(cp, "copy_kernel")
+            v = max(x[c] for x in tot.values())
+            scale[c] = (1024.0 * 1024.0) / v  # true KiB per counted unit
+            lines.append("%s on the 1 GiB copy kernel: %.0f counted -> scale factor %.4f true KiB per unit"
+                         % (c, v, scale[c]))
+        if kp:
+            tot = counter_totals(kp, "hmc_kernel")
+            big = sorted(tot.items(), key=lambda kv: -kv[1][c])[:3]
+            for disp, v in big:
+                lines.append("%s, hmc_kernel dispatch %s: %.0f counted = %.1f MiB after scaling" % (
+                    c, disp, v[c], v[c] * scale.get(c, 1.0) / 1024.0))
+    sq = find(os.path.join(out, "pmc_SQ"), "*counter_collection.csv")
+    if sq:
+        tot = counter_totals(sq, "hmc_kernel")
+        disp, v = max(tot.items(), key=lambda kv: kv[1].get("GRBM_GUI_ACTIVE", 0))
+        simd_cycles = 1024.0 * v["GRBM_GUI_ACTIVE"] / 8.0  # 8 XCDs report, 1024 SIMDs
+        lines.append("SQ counters, hmc_kernel dispatch %s (fractions of all SIMD cycles):" % disp)
+        lines.append("  MFMA pipe busy %.3f | VALU (non-MFMA) active %.3f | any instruction active %.3f | "
+                     "VALU insts per MFMA %.2f" % (
+                         v["SQ_VALU_MFMA_BUSY_CYCLES"] / simd_cycles, 4 * v["SQ_ACTIVE_INST_VALU"] / simd_cycles,
+                         4 * v["SQ_ACTIVE_INST_ANY"] / simd_cycles,
+                         (v["SQ_INSTS_VALU"] - v["SQ_INSTS_MFMA"]) / v["SQ_INSTS_MFMA"]))
+    text = "\n".join(lines)
+    print(text)
+    open(os.path.join(out, "summary.txt"), "w").write(text + "\n")
+
+
+if __name__ == "__main__":
+    main(sys.argv[1] if len(sys.argv) > 1 else "gpurun_out/profile")
