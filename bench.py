@@ -91,7 +91,8 @@ def main():
     if args.pipeline:
         launch.pipeline = args.pipeline
     wgs_per_cu = launch.wgs_per_cu if layer == pkg.LAYER_MFMA else 1
-    resident = max(1, (cus * wgs_per_cu) // launch.cus_per_chain)
+    group = launch.cus_per_chain or 8
+    resident = max(1, (cus * wgs_per_cu) // group)
     n_windows = 200 if args.full else (args.windows or resident)
 
     model = lib.default_model(lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
@@ -155,7 +156,7 @@ def main():
                         "58368x22 features ~N(0,1), teacher-MLP targets + N(0,0.01^2), Gaussian likelihood and "
                         "prior, %d leapfrog steps per transition" % (n_windows, min(n_windows, resident),
                                                                     args.leapfrog),
-            "layer": args.layer, "cus_per_chain": launch.cus_per_chain, "wgs_per_cu": wgs_per_cu,
+            "layer": args.layer, "cus_per_chain": group, "wgs_per_cu": wgs_per_cu,
             "workgroups": tm1["workgroups"], "compute_units": cus,
             "transitions_per_launch": args.transitions_per_launch,
         },

@@ -109,7 +109,9 @@ struct Plan {
   int threads = 0;
   int G = 0;
   int wgs_per_cu = 1;
-  int max_groups = 0;  // chain groups that can be co-resident
+  int max_groups = 0;  // chain groups that can be co-resident at G workgroups each
+  int resident_wgs = 0;  // workgroups that can be co-resident on the device
+  bool widen = false;    // default group size: a batch that leaves CUs idle gets wider groups
   unsigned spin_limit = 1u << 22;
   int transitions_per_launch = 8;
 };
@@ -141,8 +143,11 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
   HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, p.kernel, p.threads, 0));
   if (per_cu < 1) return fail(BNNHMC_ERR_RESIDENCY, "kernel does not fit a compute unit");
   p.wgs_per_cu = std::min(per_cu, l.wgs_per_cu);
-  p.G = l.cus_per_chain;
   const int resident = p.wgs_per_cu * di.cus;
+  p.resident_wgs = resident;
+  // 0 = default: 8 workgroups per chain (32 chains in flight on 256 CUs)
+  p.G = l.cus_per_chain > 0 ? l.cus_per_chain : std::min(8, resident);
+  p.widen = l.cus_per_chain <= 0;
   if (p.G > resident)
     return fail(BNNHMC_ERR_RESIDENCY,
                 "%d workgroups per chain requested but only %d can be resident at once", p.G,
@@ -153,33 +158,50 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
   return BNNHMC_OK;
 }
 
-size_t workspace_bytes_for(int P, int G, int groups) {
+// Exchange scratch: partial records for `wgs` co-resident workgroups (double-buffered), one totals
+// record and one barrier line per chain group (at most `groups`), status words.
+size_t workspace_bytes_for(int P, int wgs, int groups) {
   const size_t slot = (size_t)partial_slot_floats(P);
-  size_t bytes = (size_t)groups * 2 * G * slot * sizeof(float);          // partial records
-  bytes += (size_t)groups * BARRIER_STRIDE_WORDS * sizeof(unsigned);     // barrier words
-  bytes += 64 * sizeof(unsigned);                                        // status words
+  size_t bytes = (size_t)wgs * 2 * slot * sizeof(float);
+  bytes += (size_t)groups * slot * sizeof(float);
+  bytes += (size_t)groups * BARRIER_STRIDE_WORDS * sizeof(unsigned);
+  bytes += 64 * sizeof(unsigned);
   return bytes;
 }
 
 struct Workspace {
   float* partials;
+  float* totals;
   unsigned* barrier;
   unsigned* status;
 };
-Workspace carve_workspace(void* base, int P, int G, int groups) {
+Workspace carve_workspace(void* base, int P, int wgs, int groups) {
   Workspace w;
   char* b = (char*)base;
+  const size_t slot = (size_t)partial_slot_floats(P);
   w.partials = (float*)b;
-  b += (size_t)groups * 2 * G * partial_slot_floats(P) * sizeof(float);
+  b += (size_t)wgs * 2 * slot * sizeof(float);
+  w.totals = (float*)b;
+  b += (size_t)groups * slot * sizeof(float);
   w.barrier = (unsigned*)b;
   b += (size_t)groups * BARRIER_STRIDE_WORDS * sizeof(unsigned);
   w.status = (unsigned*)b;
   return w;
 }
 
+// Workgroups per chain for a batch of `groups` chains: the configured count, widened by powers of
+// two while the whole batch still fits the device (a last, smaller batch then uses every CU).
+int widen_group(int G, int groups, int resident_wgs) {
+  while (G * 2 * groups <= resident_wgs && G * 2 <= 64) G *= 2;
+  return G;
+}
+
 void set_grid(KArgs& a, int groups, int G, int* workgroups) {
   const int wgs = groups * G;
   a.G = G;
+  // measured on MI355X: up to 64 workgroups per chain the single-barrier all-read reduction is
+  // faster than two barriers with small reads (a barrier that spans XCDs costs about 10 us)
+  a.two_phase = G > 64 ? 1 : 0;
   a.n_groups = groups;
   a.xcd_map = (wgs % 8 == 0) && ((wgs / 8) % G == 0) ? 1 : 0;
   *workgroups = wgs;
@@ -288,8 +310,9 @@ KArgs base_args(const bnnhmc_sampler* s) {
   a.fixed_window = -1;
   a.L = s->hmc.leapfrog_steps;
   a.spin_limit = s->plan.spin_limit;
-  Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.G, s->plan.max_groups);
+  Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups);
   a.partials = w.partials;
+  a.totals = w.totals;
   a.barrier = w.barrier;
   a.status = w.status;
   return a;
@@ -297,7 +320,8 @@ KArgs base_args(const bnnhmc_sampler* s) {
 
 int launch_and_count(bnnhmc_sampler* s, KArgs& a, int groups) {
   int wgs = 0;
-  set_grid(a, groups, s->plan.G, &wgs);
+  set_grid(a, groups, s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs) : s->plan.G,
+           &wgs);
   HIP_TRY(launch_fill_u32(a.barrier, (size_t)groups * BARRIER_STRIDE_WORDS, 0u, s->stream));
   HIP_TRY(launch_hmc_kernel(s->plan.kernel, a, wgs, s->plan.threads, s->stream));
   s->last_workgroups = wgs;
@@ -305,7 +329,7 @@ int launch_and_count(bnnhmc_sampler* s, KArgs& a, int groups) {
 }
 
 int check_status(bnnhmc_sampler* s) {
-  Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.G, s->plan.max_groups);
+  Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups);
   unsigned st[2] = {0, 0};
   HIP_TRY(hipMemcpyAsync(st, w.status, sizeof(st), hipMemcpyDeviceToHost, s->stream));
   HIP_TRY(hipStreamSynchronize(s->stream));
@@ -372,7 +396,7 @@ void bnnhmc_default_hmc(bnnhmc_hmc* h) {
 void bnnhmc_default_launch(bnnhmc_launch* l) {
   if (!l) return;
   l->layer = BNNHMC_LAYER_MFMA;
-  l->cus_per_chain = 8;
+  l->cus_per_chain = 0;
   l->wgs_per_cu = 1;
   l->threads = 0;
   l->pipeline = 0;
@@ -429,12 +453,20 @@ float bnnhmc_rng_log_uniform(uint32_t seed, uint32_t chain_id, uint32_t t) {
 // =================================================================================================
 // operator level
 // =================================================================================================
+// workgroups the step operator gives its single chain: the configured count, or by default the
+// largest power of two that is resident at once (at most 64: wider groups are barrier-bound)
+static int step_group(const bnnhmc_launch* launch, int resident_wgs) {
+  if (launch && launch->cus_per_chain > 0) return launch->cus_per_chain;
+  int G = 1;
+  while (G * 2 <= resident_wgs && G * 2 <= 64) G *= 2;
+  return G;
+}
+
 size_t bnnhmc_step_workspace_bytes(const bnnhmc_model* model, const bnnhmc_launch* launch) {
   if (!model) return 0;
-  bnnhmc_launch l;
-  bnnhmc_default_launch(&l);
-  if (launch && launch->cus_per_chain > 0) l.cus_per_chain = launch->cus_per_chain;
-  return workspace_bytes_for(make_layout(model->d0, model->d1).P, l.cus_per_chain, 1);
+  // sized for the default group (256) when none is configured, whatever device is present
+  const int G = launch && launch->cus_per_chain > 0 ? launch->cus_per_chain : 256;
+  return workspace_bytes_for(make_layout(model->d0, model->d1).P, G, 1);
 }
 
 int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, const float* x,
@@ -455,9 +487,13 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
   rc = make_plan(*model, launch, di, plan);
   if (rc) return rc;
   const Layout L = make_layout(model->d0, model->d1);
-  if (workspace_bytes < workspace_bytes_for(L.P, plan.G, 1))
+  const int G = step_group(launch, plan.resident_wgs);
+  if (G > plan.resident_wgs)
+    return fail(BNNHMC_ERR_RESIDENCY, "%d workgroups per chain requested but only %d can be resident", G,
+                plan.resident_wgs);
+  if (workspace_bytes < workspace_bytes_for(L.P, G, 1))
     return fail(BNNHMC_ERR_INVALID, "workspace too small: %zu < %zu bytes", workspace_bytes,
-                workspace_bytes_for(L.P, plan.G, 1));
+                workspace_bytes_for(L.P, G, 1));
   hipStream_t st = (hipStream_t)stream;
   KArgs a;
   memset(&a, 0, sizeof(a));
@@ -483,12 +519,13 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
   a.ell_out = loss_values;
   a.prior_out = loss_values + model->n;
   a.spin_limit = plan.spin_limit;
-  Workspace w = carve_workspace(workspace, L.P, plan.G, 1);
+  Workspace w = carve_workspace(workspace, L.P, G, 1);
   a.partials = w.partials;
+  a.totals = w.totals;
   a.barrier = w.barrier;
   a.status = w.status;
   int wgs = 0;
-  set_grid(a, 1, plan.G, &wgs);
+  set_grid(a, 1, G, &wgs);
   // barrier and status words start from zero on every call
   HIP_TRY(launch_fill_u32(w.barrier, BARRIER_STRIDE_WORDS + 64, 0u, st));
   HIP_TRY(launch_hmc_kernel(plan.kernel, a, wgs, plan.threads, st));
@@ -498,10 +535,14 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
 int bnnhmc_step_check(const bnnhmc_model* model, const bnnhmc_launch* launch, void* workspace,
                       void* stream) {
   if (!model || !workspace) return fail(BNNHMC_ERR_INVALID, "null argument to bnnhmc_step_check");
-  bnnhmc_launch l;
-  bnnhmc_default_launch(&l);
-  if (launch && launch->cus_per_chain > 0) l.cus_per_chain = launch->cus_per_chain;
-  Workspace w = carve_workspace(workspace, make_layout(model->d0, model->d1).P, l.cus_per_chain, 1);
+  int G = launch && launch->cus_per_chain > 0 ? launch->cus_per_chain : 0;
+  if (G == 0) {
+    DeviceInfo di;
+    int rc = query_device(di);
+    if (rc) return rc;
+    G = step_group(launch, di.cus);
+  }
+  Workspace w = carve_workspace(workspace, make_layout(model->d0, model->d1).P, G, 1);
   unsigned st[2] = {0, 0};
   HIP_TRY(hipMemcpyAsync(st, w.status, sizeof(st), hipMemcpyDeviceToHost, (hipStream_t)stream));
   HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
@@ -604,7 +645,7 @@ int bnnhmc_create(const bnnhmc_model* model, const bnnhmc_hmc* hmc, const bnnhmc
   }
   const size_t C = s->n_chains;
   const int eval_groups_max = s->plan.max_groups;
-  s->workspace_bytes = workspace_bytes_for(s->L.P, s->plan.G, s->plan.max_groups);
+  s->workspace_bytes = workspace_bytes_for(s->L.P, s->plan.resident_wgs, s->plan.max_groups);
   char* ws = nullptr;
   if ((rc = s->alloc(&s->X, (size_t)n_windows * model->n * model->d0)) ||
       (rc = s->alloc(&s->y, (size_t)n_windows * s->n_pad)) ||

@@ -108,6 +108,8 @@ struct KArgs {
   uint32_t seed;
   // ---- cross-workgroup exchange ----
   float* partials;     // [group][2][G][slot]
+  float* totals;       // [group][slot]: reduced gradient, two-phase reduction only
+  int two_phase;       // 1: each workgroup reduces a slice of the parameters, then all read the totals
   unsigned* barrier;   // [group][BARRIER_STRIDE_WORDS]
   unsigned* status;    // [0] abort flag, [1] timed-out workgroup + 1
   unsigned spin_limit;

@@ -870,37 +870,98 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag);
       if (!ok) break;
       BNN_PHASE(5)  // group barrier
-      // ---- stage 2: fixed-order sum over the group's workgroups; the prior gradient seeds the sum
-      //      as block 0 does in the reference (mcmc_step_ffma.h:144) ----
       const float* grp_part = part_base + (size_t)buf * a.G * SLOT;
+      if (!a.two_phase) {
+        // ---- stage 2 (small groups): every workgroup adds the G records in rank order; the prior
+        //      gradient seeds the sum as block 0 does in the reference (mcmc_step_ffma.h:144) ----
 #pragma unroll
-      for (int i = 0; i < PPT; ++i) {
-        const int p = tid + i * T;
-        if (p < P) {
-          float v = prior_grad(mc, w[i]);
-          // eight loads in flight at a time; the additions keep the order r = 0, 1, 2, ...
-          for (int r0 = 0; r0 < a.G; r0 += 8) {
+        for (int i = 0; i < PPT; ++i) {
+          const int p = tid + i * T;
+          if (p < P) {
+            float v = prior_grad(mc, w[i]);
+            // eight loads in flight at a time; the additions keep the order r = 0, 1, 2, ...
+            for (int r0 = 0; r0 < a.G; r0 += 8) {
+              float t8[8];
+#pragma unroll
+              for (int k = 0; k < 8; ++k) {
+                const int r = r0 + k < a.G ? r0 + k : a.G - 1;
+                t8[k] = ld_agent(grp_part + (size_t)r * SLOT + p);
+              }
+#pragma unroll
+              for (int k = 0; k < 8; ++k) v += r0 + k < a.G ? t8[k] : 0.0f;
+            }
+            g[i] = v;
+          }
+        }
+        if (last) {
+          double d = 0.0;
+          for (int r = 0; r < a.G; ++r) {
+            const float lo = ld_agent(grp_part + (size_t)r * SLOT + P_AL);
+            const float hi = ld_agent(grp_part + (size_t)r * SLOT + P_AL + 1);
+            d += bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
+                                __builtin_bit_cast(uint32_t, lo));
+          }
+          dl_total = d;
+        }
+      } else {
+        // ---- stage 2 (large groups), in two phases.  Phase 1: workgroup `rank` reduces the slice
+        //      [rank S, rank S + S) of the parameters over all G records: 32 lanes per parameter, lane
+        //      `sub` adds records sub, sub + 32, ... in order, then a fixed xor tree over the 32 lanes.
+        //      Phase 2 (after a second group barrier): everyone reads the P totals. ----
+        float* tot = a.totals + (size_t)group * SLOT;
+        const int S = (P + a.G - 1) / a.G;
+        const int sub = tid & 31;
+        for (int base = 0; base < S; base += T / 32) {
+          const int pi = base + (tid >> 5);
+          const int p = rank * S + pi;
+          const bool act = pi < S && p < P;
+          const int pc = act ? p : 0;
+          float v = 0.0f;
+          for (int r0 = sub; r0 < a.G; r0 += 8 * 32) {
             float t8[8];
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
-              const int r = r0 + k < a.G ? r0 + k : a.G - 1;
-              t8[k] = ld_agent(grp_part + (size_t)r * SLOT + p);
+              const int r = r0 + 32 * k < a.G ? r0 + 32 * k : a.G - 1;
+              t8[k] = ld_agent(grp_part + (size_t)r * SLOT + pc);
             }
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v += r0 + k < a.G ? t8[k] : 0.0f;
+            for (int k = 0; k < 8; ++k) v += r0 + 32 * k < a.G ? t8[k] : 0.0f;
           }
-          g[i] = v;
+#pragma unroll
+          for (int msk = 1; msk < 32; msk <<= 1) v += __shfl_xor(v, msk);
+          if (act && sub == 0) st_agent(tot + p, v);
         }
-      }
-      if (last) {
-        double d = 0.0;
-        for (int r = 0; r < a.G; ++r) {
-          const float lo = ld_agent(grp_part + (size_t)r * SLOT + P_AL);
-          const float hi = ld_agent(grp_part + (size_t)r * SLOT + P_AL + 1);
-          d += bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
-                              __builtin_bit_cast(uint32_t, lo));
+        if (last && rank == a.G - 1 && wave == W - 1) {
+          const int lane = tid & 63;
+          double d = 0.0;
+          for (int r = lane; r < a.G; r += 64) {
+            const float lo = ld_agent(grp_part + (size_t)r * SLOT + P_AL);
+            const float hi = ld_agent(grp_part + (size_t)r * SLOT + P_AL + 1);
+            d += bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
+                                __builtin_bit_cast(uint32_t, lo));
+          }
+#pragma unroll
+          for (int msk = 1; msk < 64; msk <<= 1) d += shfl_xor_d(d, msk);
+          if (lane == 0) {
+            const uint64_t bits = double_to_bits(d);
+            st_agent(tot + P_AL, __builtin_bit_cast(float, (uint32_t)bits));
+            st_agent(tot + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)));
+          }
         }
-        dl_total = d;
+        bar_target += (unsigned)a.G;
+        ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag);
+        if (!ok) break;
+#pragma unroll
+        for (int i = 0; i < PPT; ++i) {
+          const int p = tid + i * T;
+          if (p < P) g[i] = prior_grad(mc, w[i]) + ld_agent(tot + p);
+        }
+        if (last) {
+          const float lo = ld_agent(tot + P_AL);
+          const float hi = ld_agent(tot + P_AL + 1);
+          dl_total = bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
+                                    __builtin_bit_cast(uint32_t, lo));
+        }
       }
       buf ^= 1;
       BNN_PHASE(6)  // stage 2

@@ -94,7 +94,7 @@ def test_error_codes_without_launching(pkg, lib):
     assert lib.c.bnnhmc_log_acpt(-1, 0, None, None, None, None, None, C.c_float(0), None, None, None) == pkg.ERR_INVALID
     assert lib.c.bnnhmc_sample_momentum(0, 0, 0, -1, None, None, None) == pkg.ERR_INVALID
     assert lib.c.bnnhmc_get_loss_values(None, 1, 1, None, None, None) == pkg.ERR_INVALID
-    assert lib.step_workspace_bytes(m, l) >= 2 * l.cus_per_chain * 961 * 4
+    assert lib.step_workspace_bytes(m, l) >= 2 * 256 * 961 * 4
 
 
 def test_no_device_is_reported_not_faked(pkg, lib):

@@ -63,7 +63,7 @@ def test_device_momentum_stream_is_bit_exact(lib, orc):
 @pytest.mark.parametrize("layer", ["mfma", "ffma"])
 @pytest.mark.parametrize("kind", ["t", "gauss"])
 @pytest.mark.parametrize("n,G", [(1, 1), (3, 2), (16, 1), (17, 4), (100, 3), (1000, 8), (4101, 32),
-                                 (58368, 32)])
+                                 (58368, 32), (58368, 0), (9000, 96), (58368, 256)])
 def test_eval_matches_oracle(pkg, lib, orc, layer, kind, n, G):
     say("eval layer=%s lik=%s n=%d G=%d" % (layer, kind, n, G))
     model, om, gen = models(pkg, lib, kind, n)
@@ -114,7 +114,8 @@ def test_eval_is_deterministic_and_layout_agnostic(pkg, lib, orc):
 @pytest.mark.parametrize("layer", ["mfma", "ffma"])
 @pytest.mark.parametrize("kind,n,L,eps,G", [("t", 777, 1, 0.01, 4), ("t", 2048, 2, 0.01, 8),
                                             ("t", 1500, 25, 0.01, 32), ("gauss", 999, 10, 1e-5, 5),
-                                            ("gauss", 4096, 40, 2e-5, 32)])
+                                            ("gauss", 4096, 40, 2e-5, 32), ("t", 58368, 30, 0.01, 0),
+                                            ("gauss", 20000, 12, 1e-5, 128)])
 def test_mcmc_step_operator_matches_oracle(pkg, lib, orc, layer, kind, n, L, eps, G):
     say("mcmc_step layer=%s lik=%s n=%d L=%d G=%d" % (layer, kind, n, L, G))
     model, om, gen = models(pkg, lib, kind, n)
