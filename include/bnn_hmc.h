@@ -70,10 +70,11 @@ typedef struct bnnhmc_launch {
                       /* chains in flight on 256 CUs; a smaller last batch is widened to fill the   */
                       /* device, up to 64 per chain), 64 for the step operator                      */
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */
-  int threads;        /* threads per workgroup: 256, 512, 768 or 1024 (default 1024 for MFMA,    */
+  int threads;        /* threads per workgroup: 256, 512, 768 or 1024 (default 512 for MFMA,     */
                       /* 256 for FFMA)                                                           */
-  int pipeline;       /* MFMA layer: 1 = software-pipelined tile loop (512 threads), otherwise   */
-                      /* the plain tile loop (default)                                           */
+  int pipeline;       /* MFMA tile loop: 0 or 2 = loads issued two tiles ahead with explicit     */
+                      /* waits (default), 1 = software-pipelined GEMM/pointwise stages,          */
+                      /* 3 = plain loop (default 1024 threads)                                   */
   int transitions_per_launch; /* bound on one kernel's run time (default 8)                      */
   unsigned spin_limit; /* polls before an in-kernel wait gives up (default 1 << 22)              */
 } bnnhmc_launch;
@@ -168,6 +169,13 @@ int bnnhmc_generate_window_host(uint32_t seed, uint32_t window, int n, int d0, i
 uint32_t bnnhmc_rng_word(uint32_t seed, uint32_t id, uint32_t stream, uint32_t t, uint64_t index);
 float bnnhmc_rng_normal(uint32_t seed, uint32_t id, uint32_t stream, uint32_t t, uint64_t index);
 float bnnhmc_rng_log_uniform(uint32_t seed, uint32_t chain_id, uint32_t t);
+/* Parse the reference's dataset text file (read_data, include/mcmc/io.h:43-86): one header line of
+ * total_cols tokens, then per row total_cols tokens of which the first skip_cols are ignored, the next
+ * one is the label and the next d0 are the features.  x_out[n][d0], y_out[n].  Host only.  The
+ * reference's constants are total_cols = 149, skip_cols = 2 (global_params.h:63-65); its x0.001
+ * feature scaling (main.h:162-164) is left to the caller. */
+int bnnhmc_read_reference_data(const char* path, int n, int d0, int total_cols, int skip_cols,
+                               float* x_out, float* y_out);
 /* read back a window's data (x_out[n][d0], y_out[n]; either may be NULL) */
 int bnnhmc_get_window_data(bnnhmc_sampler* s, int window, float* x_out, float* y_out);
 
@@ -186,6 +194,13 @@ int bnnhmc_get_samples(bnnhmc_sampler* s, int chain, float* samples_out, int* n_
 /* current state of one chain; any output may be NULL */
 int bnnhmc_get_chain_state(bnnhmc_sampler* s, int chain, float* w, float* grad, float* eps,
                            int* transitions_done, int* n_accepted);
+/* Overwrite the state of one chain (checkpoint resume): position w (P floats), step size, number of
+ * transitions already done (selects the RNG counters and the sample slots) and of accepted ones.  The
+ * log-posterior rows and the gradient at w are re-evaluated, which reproduces the bits a run that
+ * never stopped would hold, so the continuation is exact.  No reference counterpart (the reference
+ * keeps no checkpoint). */
+int bnnhmc_set_chain_state(bnnhmc_sampler* s, int chain, const float* w, float eps,
+                           int transitions_done, int n_accepted);
 /* per-transition traces of one chain, each of length transitions_done; any may be NULL */
 int bnnhmc_get_traces(bnnhmc_sampler* s, int chain, float* log_acpt, int* accepted, float* eps);
 

@@ -53,7 +53,7 @@ EXPORTS = [
     "bnnhmc_generate_window_host", "bnnhmc_rng_word", "bnnhmc_rng_normal", "bnnhmc_rng_log_uniform",
     "bnnhmc_get_window_data", "bnnhmc_init_chains", "bnnhmc_run", "bnnhmc_get_samples",
     "bnnhmc_get_chain_state", "bnnhmc_get_traces", "bnnhmc_eval", "bnnhmc_final_loss",
-    "bnnhmc_get_timing",
+    "bnnhmc_get_timing", "bnnhmc_read_reference_data", "bnnhmc_set_chain_state",
 ]
 
 
@@ -136,6 +136,13 @@ class Lib:
             C.c_uint32(seed), C.c_uint32(window), C.c_int(n), C.c_int(d0), C.c_int(d1),
             C.c_float(teacher_scale), C.c_float(noise_sigma), _fp(X), _fp(y), _fp(th)))
         return X, y, th
+
+    def read_reference_data(self, path, n, d0=22, total_cols=149, skip_cols=2):
+        X = np.empty((n, d0), np.float32)
+        y = np.empty(n, np.float32)
+        self.check(self.c.bnnhmc_read_reference_data(path.encode(), C.c_int(n), C.c_int(d0),
+                                                     C.c_int(total_cols), C.c_int(skip_cols), _fp(X), _fp(y)))
+        return X, y
 
     def rng_word(self, seed, id_, stream, t, index):
         return self.c.bnnhmc_rng_word(seed, id_, stream, t, index)
@@ -248,6 +255,12 @@ class Sampler:
         self.lib.check(self.lib.c.bnnhmc_get_chain_state(self.h, C.c_int(chain), _fp(w), _fp(g),
                                                          C.byref(eps), C.byref(t), C.byref(na)))
         return dict(w=w, grad=g, eps=eps.value, transitions_done=t.value, n_accepted=na.value)
+
+    def set_chain_state(self, chain, w, eps, transitions_done, n_accepted):
+        w = np.ascontiguousarray(w, np.float32)
+        assert w.shape == (self.P,)
+        self.lib.check(self.lib.c.bnnhmc_set_chain_state(self.h, C.c_int(chain), _fp(w), C.c_float(eps),
+                                                         C.c_int(transitions_done), C.c_int(n_accepted)))
 
     def get_traces(self, chain):
         T = self.hmc.burn_in + self.hmc.n_samples

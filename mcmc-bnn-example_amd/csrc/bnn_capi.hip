@@ -132,10 +132,12 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
     return fail(BNNHMC_ERR_INVALID, "unknown layer variant %d", l.layer);
   if (l.wgs_per_cu < 1 || l.wgs_per_cu > 2)
     return fail(BNNHMC_ERR_INVALID, "wgs_per_cu must be 1 or 2, got %d", l.wgs_per_cu);
-  const bool piped = l.layer == BNNHMC_LAYER_MFMA && l.pipeline == 1;
+  // MFMA tile loop: 0 / 2 = explicitly prefetched loop (default), 1 = software-pipelined, 3 = plain
+  int loop = 0;
+  if (l.layer == BNNHMC_LAYER_MFMA) loop = l.pipeline == 1 ? 1 : (l.pipeline == 3 ? 0 : 2);
   p.threads = l.threads > 0 ? l.threads
-                            : (l.layer == BNNHMC_LAYER_FFMA || l.wgs_per_cu == 2 ? 256 : (piped ? 512 : 1024));
-  p.kernel = hmc_kernel_for(m.d0, m.d1, l.layer, m.lik_kind, p.threads, piped ? 1 : 0);
+                            : (l.layer == BNNHMC_LAYER_FFMA || l.wgs_per_cu == 2 ? 256 : (loop == 0 ? 1024 : 512));
+  p.kernel = hmc_kernel_for(m.d0, m.d1, l.layer, m.lik_kind, p.threads, loop);
   if (!p.kernel)
     return fail(BNNHMC_ERR_INVALID, "no kernel for layer %d with %d threads per workgroup", l.layer,
                 p.threads);
@@ -436,6 +438,38 @@ int bnnhmc_generate_window_host(uint32_t seed, uint32_t window, int n, int d0, i
     return fail(BNNHMC_ERR_INVALID, "bad arguments to bnnhmc_generate_window_host");
   generate_window_host(seed, window, n, d0, d1, teacher_scale, noise_sigma, x_out, y_out,
                        teacher_out);
+  return BNNHMC_OK;
+}
+
+int bnnhmc_read_reference_data(const char* path, int n, int d0, int total_cols, int skip_cols,
+                               float* x_out, float* y_out) {
+  if (!path || n < 0 || d0 <= 0 || skip_cols < 0 || total_cols < skip_cols + 1 + d0 || !x_out || !y_out)
+    return fail(BNNHMC_ERR_INVALID, "bad arguments to bnnhmc_read_reference_data");
+  FILE* fp = std::fopen(path, "r");
+  if (!fp) return fail(BNNHMC_ERR_INVALID, "failed to read file '%s'", path);
+  char buf[256];
+  // the first line is a header of total_cols names (io.h:60-62)
+  for (int j = 0; j < total_cols; ++j)
+    if (std::fscanf(fp, "%255s", buf) != 1) break;
+  for (int i = 0; i < n; ++i) {
+    for (int j = 0; j < total_cols; ++j) {
+      if (std::fscanf(fp, "%255s", buf) != 1) {
+        std::fclose(fp);
+        return fail(BNNHMC_ERR_INVALID, "'%s' ends at row %d, column %d (expected %d rows of %d columns)",
+                    path, i, j, n, total_cols);
+      }
+      if (j < skip_cols || j > skip_cols + d0) continue;  // io.h:65-69
+      char* end = nullptr;
+      const float v = std::strtof(buf, &end);
+      if (end == buf) {
+        std::fclose(fp);
+        return fail(BNNHMC_ERR_INVALID, "'%s' row %d column %d is not a number: '%s'", path, i, j, buf);
+      }
+      if (j == skip_cols) y_out[i] = v;                       // io.h:71-76
+      else x_out[(size_t)i * d0 + (j - skip_cols - 1)] = v;   // io.h:77
+    }
+  }
+  std::fclose(fp);
   return BNNHMC_OK;
 }
 
@@ -867,6 +901,42 @@ int bnnhmc_get_chain_state(bnnhmc_sampler* s, int chain, float* w, float* grad, 
   if (n_accepted)
     HIP_TRY(hipMemcpyAsync(n_accepted, s->st_nacc + chain, sizeof(int), hipMemcpyDeviceToHost, s->stream));
   HIP_TRY(hipStreamSynchronize(s->stream));
+  return BNNHMC_OK;
+}
+
+int bnnhmc_set_chain_state(bnnhmc_sampler* s, int chain, const float* w, float eps,
+                           int transitions_done, int n_accepted) {
+  if (!s || !w) return fail(BNNHMC_ERR_INVALID, "null argument to bnnhmc_set_chain_state");
+  if (chain < 0 || chain >= s->n_chains)
+    return fail(BNNHMC_ERR_INVALID, "chain %d out of range [0, %d)", chain, s->n_chains);
+  if (!s->inited) return fail(BNNHMC_ERR_STATE, "bnnhmc_init_chains has not been called");
+  if (transitions_done < 0 || n_accepted < 0 || n_accepted > transitions_done)
+    return fail(BNNHMC_ERR_INVALID, "bad transition counts");
+  const size_t o = (size_t)chain * s->st_stride;
+  const int zero = 0;
+  HIP_TRY(hipMemcpyAsync(s->st_w + o, w, s->L.P * sizeof(float), hipMemcpyHostToDevice, s->stream));
+  HIP_TRY(hipMemcpyAsync(s->st_eps + chain, &eps, sizeof(float), hipMemcpyHostToDevice, s->stream));
+  HIP_TRY(hipMemcpyAsync(s->st_t + chain, &transitions_done, sizeof(int), hipMemcpyHostToDevice, s->stream));
+  HIP_TRY(hipMemcpyAsync(s->st_nacc + chain, &n_accepted, sizeof(int), hipMemcpyHostToDevice, s->stream));
+  HIP_TRY(hipMemcpyAsync(s->st_sel + chain, &zero, sizeof(int), hipMemcpyHostToDevice, s->stream));
+  HIP_TRY(hipStreamSynchronize(s->stream));
+  // gradient and per-row log-likelihood at w, exactly as the bootstrap step computes them
+  KArgs a = base_args(s);
+  a.mode = MODE_STEPS;
+  a.L = 1;
+  a.eps_in = 0.0f;
+  a.chain_base = chain;
+  a.w_in = s->st_w + o;
+  a.in_stride = s->st_stride;
+  a.g_out = s->st_g + o;
+  a.out_stride = s->st_stride;
+  a.ell_out = s->ell0 + (size_t)chain * s->n_pad;
+  a.ell_stride = s->n_pad;
+  int rc = launch_and_count(s, a, 1);
+  if (rc) return rc;
+  rc = check_status(s);
+  if (rc) return rc;
+  s->transitions_done = std::max(s->transitions_done, transitions_done);
   return BNNHMC_OK;
 }
 

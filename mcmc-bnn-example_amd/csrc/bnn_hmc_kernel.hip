@@ -421,6 +421,89 @@ struct MfmaLayer {
     }
   }
 
+  // ---- explicitly prefetched loop ----
+  // The compiler sinks ordinary loads of read-only data next to their first use, which undoes any
+  // prefetch written in the source.  Here the loads are issued by inline assembly, which it neither
+  // moves nor waits for, two tiles ahead of their use into three rotating register sets, and the
+  // waits are explicit: s_waitcnt vmcnt(14) leaves the two newer tiles (7 loads each) in flight.
+  // Memory operations the compiler adds on its own (the last step's log-likelihood rows, spills)
+  // only make these waits more conservative, never too short: vmcnt counts every outstanding
+  // operation in issue order.
+  struct TileRaw {
+    f4 xa01;   // GEMM1 operand, k-pairs 0 and 1
+    f2 xa2;    // k-pair 2 (the (1, 0) constant in lane group q = 3)
+    f2 xb[4];  // GEMM2 operand
+    f4 yv;
+  };
+  static __device__ __forceinline__ void gload2(f2& d, const float* p) {
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+  }
+  static __device__ __forceinline__ void gload4(f4& d, const float* p) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+  }
+  template <int N>
+  static __device__ __forceinline__ void wait_tile(TileRaw& t) {
+    asm volatile("s_waitcnt vmcnt(%[cnt])"
+                 : "+v"(t.xa01), "+v"(t.xa2), "+v"(t.xb[0]), "+v"(t.xb[1]), "+v"(t.xb[2]), "+v"(t.xb[3]),
+                   "+v"(t.yv)
+                 : [cnt] "n"(N)
+                 : "memory");
+  }
+
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void prefetch_loop(const StepCtx& cx, const ModelConsts& mc, int tb,
+                                                int te, int n, int q) {
+    static_assert(KP == 3, "register sets are laid out for three k-pairs");
+    const AugTable<D0>* aug = aug_table<D0>();
+    const size_t tile_floats = (size_t)16 * D0;
+    const float* pa = cx.X + (size_t)n * D0 + KS * q;
+    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
+    const float* pa_last0 = a_const ? aug->one : pa + (size_t)tb * tile_floats + 2 * (KP - 1);
+    const unsigned sa_last = a_const ? 0u : (unsigned)tile_floats;
+    const bool b_const = 2 * n >= D0;
+    const float* pb0 = b_const ? (2 * n == D0 ? aug->one : aug->zero)
+                               : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 2 * n;
+    const unsigned sb = b_const ? 0u : (unsigned)tile_floats;
+    const float* py = cx.y + 4 * q;
+    auto issue = [&](TileRaw& t, int tile) {  // exactly 7 loads
+      tile = tile < te ? tile : te - 1;
+      const unsigned rel = (unsigned)(tile - tb);
+      gload4(t.xa01, pa + (size_t)tile * tile_floats);
+      gload2(t.xa2, pa_last0 + (size_t)rel * sa_last);
+      const float* rb = pb0 + (size_t)rel * sb;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) gload2(t.xb[j], rb + j * D0);
+      gload4(t.yv, py + (size_t)tile * 16);
+    };
+    auto compute = [&](TileRaw& t, int tile) {
+      wait_tile<14>(t);
+      const f2 xa[KP] = {f2{t.xa01[0], t.xa01[1]}, f2{t.xa01[2], t.xa01[3]}, t.xa2};
+      f4 acc[NT];
+      gemm1(xa, acc);
+      pointwise<LIK, LAST, true>(acc, t.yv, cx, mc, tile * 16, n, q);
+      gemm2(acc, t.xb);
+    };
+    TileRaw A, B, C;
+    issue(A, tb);
+    issue(B, tb + 1);
+    for (int i = tb; i < te; i += 3) {
+      issue(C, i + 2);
+      compute(A, i);
+      if (i + 1 < te) {
+        issue(A, i + 3);
+        compute(B, i + 1);
+      }
+      if (i + 2 < te) {
+        issue(B, i + 4);
+        compute(C, i + 2);
+      }
+    }
+    // no register of a set may be reused before its last load has landed
+    wait_tile<0>(A);
+    wait_tile<0>(B);
+    wait_tile<0>(C);
+  }
+
   template <int LIK, bool LAST>
   __device__ __forceinline__ void run_tiles(const StepCtx& cx, const ModelConsts& mc) {
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
@@ -428,7 +511,8 @@ struct MfmaLayer {
     int fast_end = tb;
     if (cx.x_vec_ok && cx.y_vec_ok) fast_end = min(te, cx.n / 16);
     if (fast_end > tb) {
-      if (PIPE) fast_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
+      if (PIPE == 1) fast_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
+      else if (PIPE == 2) prefetch_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
       else simple_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
     }
     // ragged tail tile, or unaligned caller buffers: one tile at a time
@@ -1100,8 +1184,13 @@ const void* hmc_kernel_for(int d0, int d1, int layer, int lik, int threads, int 
   if (d0 != 22 || d1 != 40) return nullptr;
   using MP = MfmaLayer<22, 40, 1>;
   using MS = MfmaLayer<22, 40, 0>;
+  using MA = MfmaLayer<22, 40, 2>;
   using F = FfmaLayer<22, 40>;
-  if (layer == 0 && pipeline) {
+  if (layer == 0 && pipeline == 2) {
+    if (threads == 1024) return lik == 0 ? kernel_ptr<MA, 0, 1024>() : kernel_ptr<MA, 1, 1024>();
+    if (threads == 768) return lik == 0 ? kernel_ptr<MA, 0, 768>() : kernel_ptr<MA, 1, 768>();
+    if (threads == 512) return lik == 0 ? kernel_ptr<MA, 0, 512>() : kernel_ptr<MA, 1, 512>();
+  } else if (layer == 0 && pipeline == 1) {
     if (threads == 512) return lik == 0 ? kernel_ptr<MP, 0, 512>() : kernel_ptr<MP, 1, 512>();
     if (threads == 256) return lik == 0 ? kernel_ptr<MP, 0, 256>() : kernel_ptr<MP, 1, 256>();
   } else if (layer == 0) {

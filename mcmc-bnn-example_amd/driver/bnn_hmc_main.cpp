@@ -62,33 +62,6 @@ bool parse(int argc, char** argv, Options& o) {
   return true;
 }
 
-// the reference's dataset format (include/mcmc/io.h:43-86): one header line of 149 tokens, then per
-// row 149 columns of which the first 2 are skipped, the next is the label and the next 22 the features
-bool read_reference_data(const std::string& path, int rows, std::vector<float>& x, std::vector<float>& y) {
-  const int total_cols = 149, skip = 2, d0 = 22;
-  FILE* fp = std::fopen(path.c_str(), "r");
-  if (!fp) return false;
-  char buf[256];
-  for (int j = 0; j < total_cols; ++j)
-    if (std::fscanf(fp, "%255s", buf) == EOF) break;
-  x.assign((size_t)rows * d0, 0.0f);
-  y.assign(rows, 0.0f);
-  for (int i = 0; i < rows; ++i) {
-    for (int j = 0; j < total_cols; ++j) {
-      if (std::fscanf(fp, "%255s", buf) == EOF) {
-        std::fclose(fp);
-        return false;
-      }
-      if (j < skip || j >= skip + 1 + d0) continue;
-      const float v = std::strtof(buf, nullptr);
-      if (j == skip) y[i] = v;
-      else x[(size_t)i * d0 + (j - skip - 1)] = v;
-    }
-  }
-  std::fclose(fp);
-  return true;
-}
-
 // shape / min / max / mean summary the reference prints for a matrix (utils_matrix.h:160-178)
 void print_stats(const char* name, const float* d, size_t rows, size_t cols) {
   float mn = INFINITY, mx = -INFINITY, mean = 0.0f;
@@ -140,12 +113,9 @@ int main(int argc, char** argv) {
   CHECK(bnnhmc_create(&model, &hmc, &launch, o.windows, o.chains, &s));
   const int P = bnnhmc_num_params(model.d0, model.d1);
   if (!o.data.empty()) {
-    std::vector<float> x, y;
+    std::vector<float> x((size_t)model.n * model.d0), y(model.n);
     std::printf("Reading dataset...\n");
-    if (!read_reference_data(o.data, model.n, x, y)) {
-      std::fprintf(stderr, "Error: failed to read file '%s'!\n", o.data.c_str());
-      return 1;
-    }
+    CHECK(bnnhmc_read_reference_data(o.data.c_str(), model.n, model.d0, 149, 2, x.data(), y.data()));
     std::printf("Dataset read successfully\n");
     print_stats("Data", x.data(), model.n, model.d0);
     print_stats("Labels", y.data(), model.n, 1);

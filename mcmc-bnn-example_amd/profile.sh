@@ -5,7 +5,7 @@
 # Usage: bash mcmc-bnn-example_amd/profile.sh [extra bench.py arguments]
 set -e
 ROOT="$(cd "$(dirname "$0")/.." && pwd)"
-OUT="$ROOT/gpurun_out/profile"
+OUT="$ROOT/gpurun_out/${PROFILE_DIR:-profile}"
 mkdir -p "$OUT"
 BENCH_ARGS="--steps 10 --warmup 5 --cpu-seconds 0 $*"
 cd /tmp && export TMPDIR=/tmp
@@ -24,4 +24,7 @@ echo "== SQ counters (trajectory kernel)"
 timeout -s KILL 300 rocprofv3 --pmc SQ_BUSY_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_ACTIVE_INST_VALU SQ_INSTS_VALU \
   SQ_INSTS_MFMA SQ_WAIT_INST_ANY SQ_WAVE_CYCLES SQ_ACTIVE_INST_ANY GRBM_GUI_ACTIVE -d "$OUT/pmc_SQ" -o pmc \
   --output-format csv -- python3 "$ROOT/bench.py" $BENCH_ARGS > "$OUT/bench_SQ.json" 2> "$OUT/pmc_SQ.log"
+echo "== L2 counters (trajectory kernel)"
+timeout -s KILL 300 rocprofv3 --pmc TCC_HIT_sum TCC_MISS_sum TCC_EA0_RDREQ_sum TCC_EA0_RDREQ_DRAM_sum -d "$OUT/pmc_TCC" -o pmc \
+  --output-format csv -- python3 "$ROOT/bench.py" $BENCH_ARGS > "$OUT/bench_TCC.json" 2> "$OUT/pmc_TCC.log"
 python3 "$ROOT/mcmc-bnn-example_amd/profile_summary.py" "$OUT"

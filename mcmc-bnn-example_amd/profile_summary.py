@@ -76,7 +76,15 @@ def main(out):
                      "VALU insts per MFMA %.2f" % (
                          v["SQ_VALU_MFMA_BUSY_CYCLES"] / simd_cycles, 4 * v["SQ_ACTIVE_INST_VALU"] / simd_cycles,
                          4 * v["SQ_ACTIVE_INST_ANY"] / simd_cycles,
-                         (v["SQ_INSTS_VALU"] - v["SQ_INSTS_MFMA"]) / v["SQ_INSTS_MFMA"]))
+                         (v["SQ_INSTS_VALU"] - v["SQ_INSTS_MFMA"]) / max(1.0, v["SQ_INSTS_MFMA"])))
+    tcc = find(os.path.join(out, "pmc_TCC"), "*counter_collection.csv")
+    if tcc:
+        tot = counter_totals(tcc, "hmc_kernel")
+        disp, v = max(tot.items(), key=lambda kv: kv[1].get("TCC_HIT_sum", 0) + kv[1].get("TCC_MISS_sum", 0))
+        hit, miss = v["TCC_HIT_sum"], v["TCC_MISS_sum"]
+        lines.append("L2 (TCC), hmc_kernel dispatch %s: hits %.4g, misses %.4g -> hit rate %.3f; read requests to "
+                     "the fabric %.4g of which marked DRAM %.4g" % (disp, hit, miss, hit / max(1.0, hit + miss),
+                                                                   v["TCC_EA0_RDREQ_sum"], v["TCC_EA0_RDREQ_DRAM_sum"]))
     text = "\n".join(lines)
     print(text)
     open(os.path.join(out, "summary.txt"), "w").write(text + "\n")

@@ -106,3 +106,25 @@ def test_no_device_is_reported_not_faked(pkg, lib):
     hnd = C.c_void_p()
     assert lib.c.bnnhmc_create(C.byref(m), C.byref(h), C.byref(l), 1, 1, C.byref(hnd)) == pkg.ERR_NO_DEVICE
     assert not hnd.value
+
+
+def test_reference_text_reader(lib, pkg, tmp_path):
+    # the reference's file layout (io.h:43-86): header line, then 149 columns per row of which the
+    # first 2 are skipped, column 2 is the label and columns 3..24 are the 22 features
+    rng = np.random.default_rng(0)
+    n, cols = 7, 149
+    table = rng.normal(0, 3, (n, cols)).round(4)
+    path = tmp_path / "returns_and_features_for_mcmc.txt"
+    with open(path, "w") as f:
+        f.write(" ".join("col%d" % j for j in range(cols)) + "\n")
+        for i in range(n):
+            f.write(" ".join(["2020-01-%02d" % (i + 1), "ID%d" % i] + ["%.4f" % v for v in table[i, 2:]]) + "\n")
+    X, y = lib.read_reference_data(str(path), n)
+    np.testing.assert_array_equal(y, table[:, 2].astype(np.float32))
+    np.testing.assert_array_equal(X, table[:, 3:25].astype(np.float32))
+    # a short file and a missing file are errors, not aborts
+    with pytest.raises(pkg.BnnHmcError) as e:
+        lib.read_reference_data(str(path), n + 1)
+    assert e.value.code == pkg.ERR_INVALID and "ends at row" in str(e.value)
+    with pytest.raises(pkg.BnnHmcError):
+        lib.read_reference_data(str(tmp_path / "missing.txt"), n)

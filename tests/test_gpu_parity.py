@@ -322,3 +322,93 @@ def test_residency_and_timeout_are_reported(pkg, lib):
     with pytest.raises(pkg.BnnHmcError) as e:
         lib.create(m, lib.default_hmc(), lib.default_launch(cus_per_chain=100000), 1, 1)
     assert e.value.code == pkg.ERR_RESIDENCY
+
+
+def test_posterior_moments_over_800_samples(pkg, lib, orc):
+    """Posterior mean / std of every weight over 800 kept samples agree with the oracle's chain within
+    the Monte-Carlo error of those estimates.  The two chains share the RNG stream and take identical
+    decisions at first; FP32 rounding eventually flips one and they become two realisations of the
+    same sampler, so the comparison is statistical: batch-means standard errors (valid here: the
+    posterior is chosen so that HMC mixes within a few transitions -- two oracle chains with different
+    seeds give max z = 3.2 over the 961 weights and std ratios in [0.86, 1.18])."""
+    say("posterior moments, 900 transitions")
+    n, L, burn, keep = 256, 25, 100, 800
+    model = lib.default_model(n=n, lik_scale=1.0, prior_scale=0.3)
+    om = ob.Model(D0, D1, n, ob.LIK_STUDENT_T, 1.0, 2.2, 0.3)
+    hmc = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=0.01, seed=33)
+    s = lib.create(model, hmc, lib.default_launch(cus_per_chain=4, transitions_per_launch=50), 1, 1)
+    s.generate_window(0, teacher_scale=0.3, noise_sigma=1.0)
+    X, y = s.get_window_data(0)
+    s.init_chains(None)
+    s.run(burn + keep)
+    a = s.get_samples(0).astype(np.float64)
+    tr = s.get_traces(0)
+    s.close()
+    ref = orc.run_chain(om, ob.Hmc(L, burn, keep, burn, 0.01, 0.2, 0.1, 0.01, 33, 0), X, y)
+    b = ref["samples"].astype(np.float64)
+    assert a.shape == b.shape == (keep, P)
+    assert np.array_equal(tr["accept"][:50], ref["accept"][:50])
+    assert abs(tr["accept"].mean() - ref["accept"].mean()) < 0.05
+
+    def batch_means_se(x, nb=20):
+        bm = x.reshape(nb, -1, x.shape[1]).mean(1)
+        return bm.std(0, ddof=1) / math.sqrt(nb)
+
+    se = np.sqrt(batch_means_se(a) ** 2 + batch_means_se(b) ** 2)   # Monte-Carlo error of a difference
+    z = np.abs(a.mean(0) - b.mean(0)) / se
+    assert z.max() < 5.0, "a posterior mean is off by %.2f Monte-Carlo standard errors" % z.max()
+    assert np.mean(z > 3.0) < 0.02
+    ratio = a.std(0) / b.std(0)
+    assert 0.75 < ratio.min() and ratio.max() < 1.33
+
+
+def test_resume_from_saved_state_is_exact(pkg, lib, orc):
+    n, L, burn, keep = 1200, 10, 4, 12
+    model, om, gen = models(pkg, lib, "t_stiff", n)
+    hmc = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=0.01, seed=5)
+    launch = lib.default_launch(cus_per_chain=4, transitions_per_launch=3)
+
+    def fresh():
+        s = lib.create(model, hmc, launch, 1, 2)
+        s.generate_window(0, **gen)
+        s.init_chains(None)
+        return s
+
+    s = fresh()
+    s.run(burn + keep)
+    full = [s.get_samples(c) for c in range(2)]
+    full_state = [s.get_chain_state(c) for c in range(2)]
+    s.close()
+    s = fresh()
+    s.run(9)
+    saved = [s.get_chain_state(c) for c in range(2)]
+    s.close()
+    s = fresh()                                    # a new sampler, as after a restart
+    for c in range(2):
+        st = saved[c]
+        s.set_chain_state(c, st["w"], st["eps"], st["transitions_done"], st["n_accepted"])
+    s.run(burn + keep - 9)
+    for c in range(2):
+        got = s.get_samples(c)
+        assert got[9 - burn:].tobytes() == full[c][9 - burn:].tobytes()
+        st = s.get_chain_state(c)
+        assert st["w"].tobytes() == full_state[c]["w"].tobytes()
+        assert st["grad"].tobytes() == full_state[c]["grad"].tobytes()
+        assert st["eps"] == full_state[c]["eps"] and st["n_accepted"] == full_state[c]["n_accepted"]
+    s.close()
+
+
+def test_host_driver_runs_init_run_dump(pkg, tmp_path):
+    import os
+    import subprocess
+
+    exe = os.path.join(pkg.PKG_DIR, "bnn_hmc_main")
+    assert os.path.exists(exe), "driver not built"
+    dump = tmp_path / "chain.bin"
+    r = subprocess.run([exe, "--windows", "2", "--rows", "2048", "--samples", "6", "--burn-in", "4",
+                        "--leapfrog", "20", "--dump", str(dump)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "Final samples: Shape: 6 x 961" in r.stdout and "Final loss1:" in r.stdout
+    assert "MCMC (4 burn in, 6 sample steps, 20 leap-frog steps) done in" in r.stdout
+    data = np.fromfile(dump, np.float32)
+    assert data.size == 2 * 6 * 961 and np.all(np.isfinite(data))
