@@ -29,7 +29,7 @@ EVALS_200x1600 = 200 * (1700 * 1000 + 1)
 # HBM-side bytes per gradient evaluation of the MFMA trajectory kernel, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE scaled by a 1 GiB copy kernel (profiles/hmc_kernel_mfma_22x40_32windows.txt): one window's
 # X and y (5.37 MB) pass through L2 once per leapfrog step, plus the partial-gradient records.
-TRAFFIC_BYTES_PER_EVAL_MFMA = 9.388e11 / 160000
+TRAFFIC_BYTES_PER_EVAL_MFMA = 8.697e11 / 160000
 
 
 def cpu_baseline(seconds):
@@ -91,7 +91,7 @@ def main():
     if args.pipeline:
         launch.pipeline = args.pipeline
     wgs_per_cu = launch.wgs_per_cu if layer == pkg.LAYER_MFMA else 1
-    group = launch.cus_per_chain or 8
+    group = launch.cus_per_chain or 4
     resident = max(1, (cus * wgs_per_cu) // group)
     n_windows = 200 if args.full else (args.windows or resident)
 

@@ -66,7 +66,7 @@ typedef struct bnnhmc_hmc {
 /* How the work is laid over the GPU.  Zero in a field selects the default. */
 typedef struct bnnhmc_launch {
   int layer;          /* BNNHMC_LAYER_MFMA (v_mfma_f32_16x16x4_f32) or BNNHMC_LAYER_FFMA          */
-  int cus_per_chain;  /* workgroups that share one chain's rows; 0 = default: 8 for a sampler (32   */
+  int cus_per_chain;  /* workgroups that share one chain's rows; 0 = default: 4 for a sampler (64   */
                       /* chains in flight on 256 CUs; a smaller last batch is widened to fill the   */
                       /* device, up to 64 per chain), 64 for the step operator                      */
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */

@@ -147,8 +147,8 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
   p.wgs_per_cu = std::min(per_cu, l.wgs_per_cu);
   const int resident = p.wgs_per_cu * di.cus;
   p.resident_wgs = resident;
-  // 0 = default: 8 workgroups per chain (32 chains in flight on 256 CUs)
-  p.G = l.cus_per_chain > 0 ? l.cus_per_chain : std::min(8, resident);
+  // 0 = default: 4 workgroups per chain (64 chains in flight on 256 CUs)
+  p.G = l.cus_per_chain > 0 ? l.cus_per_chain : std::min(4, resident);
   p.widen = l.cus_per_chain <= 0;
   if (p.G > resident)
     return fail(BNNHMC_ERR_RESIDENCY,
@@ -207,6 +207,14 @@ void set_grid(KArgs& a, int groups, int G, int* workgroups) {
   a.n_groups = groups;
   a.xcd_map = (wgs % 8 == 0) && ((wgs / 8) % G == 0) ? 1 : 0;
   *workgroups = wgs;
+}
+
+// Test hook: BNNHMC_DEBUG_DROP_ARRIVAL=<rank> makes that rank of every chain group withhold its
+// arrival at the group barrier, so that the bounded wait of the others expires (every workgroup still
+// exits normally).  Unset in normal use.
+int debug_drop_rank() {
+  const char* e = getenv("BNNHMC_DEBUG_DROP_ARRIVAL");
+  return e && *e ? atoi(e) : -1;
 }
 
 // host restatement of the hidden activation (kernel_helpers.h:34-42) for the data generator
@@ -312,6 +320,7 @@ KArgs base_args(const bnnhmc_sampler* s) {
   a.fixed_window = -1;
   a.L = s->hmc.leapfrog_steps;
   a.spin_limit = s->plan.spin_limit;
+  a.debug_drop_rank = debug_drop_rank();
   Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups);
   a.partials = w.partials;
   a.totals = w.totals;
@@ -553,6 +562,7 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
   a.ell_out = loss_values;
   a.prior_out = loss_values + model->n;
   a.spin_limit = plan.spin_limit;
+  a.debug_drop_rank = debug_drop_rank();
   Workspace w = carve_workspace(workspace, L.P, G, 1);
   a.partials = w.partials;
   a.totals = w.totals;

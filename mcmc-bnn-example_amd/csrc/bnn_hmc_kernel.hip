@@ -745,11 +745,11 @@ struct FfmaLayer {
 // launch is abandoned (status[0] set), so every wave always exits.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ bool group_barrier(unsigned* counter, unsigned target, unsigned* status,
-                                              unsigned spin_limit, int* s_flag) {
+                                              unsigned spin_limit, int* s_flag, bool signal = true) {
   __syncthreads();  // this workgroup's partials are stored (and waited for)
   if (threadIdx.x == 0) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (signal) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     unsigned polls = 0;
     int ok = 1;
     while ((int)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
@@ -951,7 +951,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       }
       BNN_PHASE(4)  // stage 1 + global store
       bar_target += (unsigned)a.G;
-      ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag);
+      ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag, rank != a.debug_drop_rank);
       if (!ok) break;
       BNN_PHASE(5)  // group barrier
       const float* grp_part = part_base + (size_t)buf * a.G * SLOT;
@@ -1033,7 +1033,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
           }
         }
         bar_target += (unsigned)a.G;
-        ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag);
+        ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag, rank != a.debug_drop_rank);
         if (!ok) break;
 #pragma unroll
         for (int i = 0; i < PPT; ++i) {

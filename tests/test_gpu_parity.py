@@ -317,11 +317,30 @@ def test_full_size_properties(pkg, lib, orc):
     close_grad(halves[0] + halves[1] - prior_g, g_all.astype(np.float64), "additivity", rtol=3e-6)
 
 
-def test_residency_and_timeout_are_reported(pkg, lib):
+def test_residency_and_timeout_are_reported(pkg, lib, orc, monkeypatch):
     m = lib.default_model(n=64)
     with pytest.raises(pkg.BnnHmcError) as e:
         lib.create(m, lib.default_hmc(), lib.default_launch(cus_per_chain=100000), 1, 1)
     assert e.value.code == pkg.ERR_RESIDENCY
+    # a workgroup that never arrives at the group barrier: the others' bounded wait expires, every
+    # workgroup exits, the call reports BNNHMC_ERR_TIMEOUT and the sampler stays usable
+    n = 4096
+    model, om, gen = models(pkg, lib, "t", n)
+    s = lib.create(model, lib.default_hmc(leapfrog_steps=5, burn_in=2, n_samples=2),
+                   lib.default_launch(cus_per_chain=4, spin_limit=4096), 1, 1)
+    th = s.generate_window(0, **gen)
+    X, y = s.get_window_data(0)
+    monkeypatch.setenv("BNNHMC_DEBUG_DROP_ARRIVAL", "2")
+    with pytest.raises(pkg.BnnHmcError) as e:
+        s.eval(0, th)
+    assert e.value.code == pkg.ERR_TIMEOUT and "spin limit" in str(e.value)
+    monkeypatch.delenv("BNNHMC_DEBUG_DROP_ARRIVAL")
+    _, _, grad = s.eval(0, th)
+    close_grad(grad, orc.eval_f32(om, X, y, th)[2].astype(np.float64), "after a timed-out launch")
+    s.init_chains(None)
+    s.run(4)
+    assert s.get_chain_state(0)["transitions_done"] == 4
+    s.close()
 
 
 def test_posterior_moments_over_800_samples(pkg, lib, orc):
