@@ -14,104 +14,11 @@
 #include <hip/hip_runtime.h>
 
 #include "bnn_device.h"
+#include "bnn_kernel_common.h"
 #include "bnn_kernels.h"
 #include "bnn_rng.h"
 
 namespace bnn {
-
-typedef float f4 __attribute__((ext_vector_type(4)));
-typedef float f2 __attribute__((ext_vector_type(2)));
-
-// ------------------------------------------------------------------------------------------------
-// small device helpers
-// ------------------------------------------------------------------------------------------------
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-  return __builtin_bit_cast(
-      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
-}
-
-// sum over the 16 lanes of a DPP row; every lane of the row receives the same bits (each step adds
-// a value to its mirror image, and a + b == b + a)
-__device__ __forceinline__ float row16_allreduce(float v) {
-  v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
-  v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
-  v += dpp_move<0x141>(v);  // row_half_mirror
-  v += dpp_move<0x140>(v);  // row_mirror
-  return v;
-}
-// sum over the 8 lanes of a half row
-__device__ __forceinline__ float row8_allreduce(float v) {
-  v += dpp_move<0xB1>(v);
-  v += dpp_move<0x4E>(v);
-  v += dpp_move<0x141>(v);
-  return v;
-}
-
-__device__ __forceinline__ double shfl_xor_d(double v, int mask) {
-  const uint64_t b = double_to_bits(v);
-  const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)b, mask);
-  const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(b >> 32), mask);
-  return bits_to_double(((uint64_t)hi << 32) | lo);
-}
-
-// activation of the hidden layer, include/mcmc/kernel_helpers.h:34-42:
-// tanh(x) = 2 sigmoid(2x) - 1 with e^(-2x) = 2^(x * -2/ln 2); identity below the cutoff
-__device__ __forceinline__ float tanh_fwd(float x) {
-  const float e = __builtin_amdgcn_exp2f(x * -2.88539008177792681472f);
-  const float sigm = __builtin_amdgcn_rcpf(1.0f + e);
-  const float r = __builtin_fmaf(sigm, 2.0f, -1.0f);
-  return __builtin_fabsf(x) < 0.0048176045529544353485f ? x : r;
-}
-
-// per-row log-likelihood gradient (and value) given the residual, mcmc_step_ffma.h:293-301
-template <int LIK>
-__device__ __forceinline__ float lik_grad(const ModelConsts& mc, float resid, float& diff_out) {
-  const float diff = resid * mc.scale_recp;
-  diff_out = diff;
-  if (LIK == 0) {
-    return diff * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(diff, diff, mc.df));
-  } else {
-    return diff * mc.scale_recp;
-  }
-}
-template <int LIK>
-__device__ __forceinline__ float lik_value(const ModelConsts& mc, float diff) {
-  if (LIK == 0) {
-    return mc.l_scale * log1pf(diff * diff * mc.df_recp) - mc.lik_norm;
-  } else {
-    return -0.5f * (diff * diff) - mc.lik_norm;
-  }
-}
-
-// prior terms, mcmc_step_ffma.h:113-118
-__device__ __forceinline__ float prior_logp(const ModelConsts& mc, float w) {
-  const float lp = w * mc.prior_recp;
-  return -(lp * lp) * 0.5f - mc.prior_norm;
-}
-__device__ __forceinline__ float prior_grad(const ModelConsts& mc, float w) {
-  return w * mc.prior_neg_recp2;
-}
-
-__device__ __forceinline__ float ld_agent(const float* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void st_agent(float* p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// ------------------------------------------------------------------------------------------------
-// Per-wave working set handed to a layer for one leapfrog step
-// ------------------------------------------------------------------------------------------------
-struct StepCtx {
-  const float* X;        // this window's rows
-  const float* y;
-  int n;
-  int tile_begin, tile_end;  // 16-row tiles of this wave
-  bool x_vec_ok, y_vec_ok;
-  const float* ell_prev;  // last step only: rows of the current state (null = zeros)
-  float* ell_new;         // last step only: where to store this state's rows (null = skip)
-};
 
 // Constant operand slots of the MFMA layer: `one` reads (1, 0) at offsets j * D0 (j < 4), `zero` reads
 // (0, 0); lanes holding the appended constant-one feature or tile padding point here.
@@ -738,42 +645,6 @@ struct FfmaLayer {
     }
   }
 };
-
-// ------------------------------------------------------------------------------------------------
-// group barrier: all G workgroups of a chain group have published their partials of this step.
-// Bounded: after spin_limit polls, or when another workgroup has given up, the wait ends and the
-// launch is abandoned (status[0] set), so every wave always exits.
-// ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ bool group_barrier(unsigned* counter, unsigned target, unsigned* status,
-                                              unsigned spin_limit, int* s_flag, bool signal = true) {
-  __syncthreads();  // this workgroup's partials are stored (and waited for)
-  if (threadIdx.x == 0) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    if (signal) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    unsigned polls = 0;
-    int ok = 1;
-    while ((int)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
-      __builtin_amdgcn_s_sleep(2);
-      if ((++polls & 63u) == 0u) {
-        if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
-          ok = 0;
-          break;
-        }
-        if (polls >= spin_limit) {
-          __hip_atomic_store(status + 1, (unsigned)blockIdx.x + 1u, __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_AGENT);
-          __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          ok = 0;
-          break;
-        }
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    *s_flag = ok;
-  }
-  __syncthreads();
-  return *s_flag != 0;
-}
 
 // ------------------------------------------------------------------------------------------------
 // the kernel
