@@ -65,9 +65,10 @@ ModelConsts make_consts(const bnnhmc_model& m) {
 
 int check_model(const bnnhmc_model* m) {
   if (!m) return fail(BNNHMC_ERR_INVALID, "model is null");
-  if (m->d0 != 22 || m->d1 != 40)
-    return fail(BNNHMC_ERR_INVALID, "unsupported layer sizes %d -> %d -> 1 (built: 22 -> 40 -> 1)",
-                m->d0, m->d1);
+  if (!(m->d0 == 22 && m->d1 == 40) && !(m->d0 == 64 && m->d1 == 128))
+    return fail(BNNHMC_ERR_INVALID,
+                "unsupported layer sizes %d -> %d -> 1 (built: 22 -> 40 -> 1 and 64 -> 128 -> 1)", m->d0,
+                m->d1);
   if (m->n <= 0) return fail(BNNHMC_ERR_INVALID, "n must be positive, got %d", m->n);
   if (m->lik_kind != BNNHMC_LIK_STUDENT_T && m->lik_kind != BNNHMC_LIK_GAUSSIAN)
     return fail(BNNHMC_ERR_INVALID, "unknown likelihood kind %d", m->lik_kind);
@@ -107,6 +108,9 @@ int query_device(DeviceInfo& di) {
 struct Plan {
   const void* kernel = nullptr;
   int threads = 0;
+  bool wide = false;             // LDS-resident parameter kernel (64 -> 128 -> 1)
+  size_t dyn_lds = 0;            // dynamic LDS bytes per workgroup
+  size_t wg_scratch_floats = 0;  // private global scratch per workgroup (transitions only)
   int G = 0;
   int wgs_per_cu = 1;
   int max_groups = 0;  // chain groups that can be co-resident at G workgroups each
@@ -135,14 +139,27 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
   // MFMA tile loop: 0 / 2 = explicitly prefetched loop (default), 1 = software-pipelined, 3 = plain
   int loop = 0;
   if (l.layer == BNNHMC_LAYER_MFMA) loop = l.pipeline == 1 ? 1 : (l.pipeline == 3 ? 0 : 2);
-  p.threads = l.threads > 0 ? l.threads
-                            : (l.layer == BNNHMC_LAYER_FFMA || l.wgs_per_cu == 2 ? 256 : (loop == 0 ? 1024 : 512));
-  p.kernel = hmc_kernel_for(m.d0, m.d1, l.layer, m.lik_kind, p.threads, loop);
+  p.wide = m.d0 == 64 && m.d1 == 128;
+  if (p.wide) {
+    if (l.layer != BNNHMC_LAYER_MFMA)
+      return fail(BNNHMC_ERR_INVALID, "64 -> 128 -> 1 is built for the MFMA layer only");
+    if (l.cus_per_chain > 64)
+      return fail(BNNHMC_ERR_INVALID, "64 -> 128 -> 1 supports at most 64 workgroups per chain, got %d",
+                  l.cus_per_chain);
+    p.threads = l.threads > 0 ? l.threads : 256;
+    p.kernel = hmc_kernel_wide_for(m.d0, m.d1, m.lik_kind, p.threads, &p.dyn_lds, &p.wg_scratch_floats);
+  } else {
+    p.threads = l.threads > 0 ? l.threads
+                              : (l.layer == BNNHMC_LAYER_FFMA || l.wgs_per_cu == 2 ? 256 : (loop == 0 ? 1024 : 512));
+    p.kernel = hmc_kernel_for(m.d0, m.d1, l.layer, m.lik_kind, p.threads, loop);
+  }
   if (!p.kernel)
     return fail(BNNHMC_ERR_INVALID, "no kernel for layer %d with %d threads per workgroup", l.layer,
                 p.threads);
+  if (p.dyn_lds > 0)
+    HIP_TRY(hipFuncSetAttribute(p.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)p.dyn_lds));
   int per_cu = 0;
-  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, p.kernel, p.threads, 0));
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, p.kernel, p.threads, p.dyn_lds));
   if (per_cu < 1) return fail(BNNHMC_ERR_RESIDENCY, "kernel does not fit a compute unit");
   p.wgs_per_cu = std::min(per_cu, l.wgs_per_cu);
   const int resident = p.wgs_per_cu * di.cus;
@@ -278,6 +295,7 @@ struct bnnhmc_sampler {
   float* tr_eps = nullptr;
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
+  float* wg_scratch = nullptr;  // wide-layer kernel: per-workgroup accepted state and start momentum
   float* tmp = nullptr;       // evaluation scratch: w | grad | prior (3 * st_stride) ...
   float* tmp_ell = nullptr;   // ... and n_pad rows
   double* tmp_sums = nullptr; // [max_groups][2]
@@ -326,6 +344,7 @@ KArgs base_args(const bnnhmc_sampler* s) {
   a.totals = w.totals;
   a.barrier = w.barrier;
   a.status = w.status;
+  a.wg_scratch = s->wg_scratch;
   return a;
 }
 
@@ -334,7 +353,7 @@ int launch_and_count(bnnhmc_sampler* s, KArgs& a, int groups) {
   set_grid(a, groups, s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs) : s->plan.G,
            &wgs);
   HIP_TRY(launch_fill_u32(a.barrier, (size_t)groups * BARRIER_STRIDE_WORDS, 0u, s->stream));
-  HIP_TRY(launch_hmc_kernel(s->plan.kernel, a, wgs, s->plan.threads, s->stream));
+  HIP_TRY(launch_hmc_kernel(s->plan.kernel, a, wgs, s->plan.threads, s->plan.dyn_lds, s->stream));
   s->last_workgroups = wgs;
   return BNNHMC_OK;
 }
@@ -534,6 +553,8 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
   if (G > plan.resident_wgs)
     return fail(BNNHMC_ERR_RESIDENCY, "%d workgroups per chain requested but only %d can be resident", G,
                 plan.resident_wgs);
+  if (plan.wide && G > 64)
+    return fail(BNNHMC_ERR_INVALID, "64 -> 128 -> 1 supports at most 64 workgroups per chain, got %d", G);
   if (workspace_bytes < workspace_bytes_for(L.P, G, 1))
     return fail(BNNHMC_ERR_INVALID, "workspace too small: %zu < %zu bytes", workspace_bytes,
                 workspace_bytes_for(L.P, G, 1));
@@ -545,7 +566,8 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
   a.mc = make_consts(*model);
   a.X = x;
   a.y = y;
-  a.x_vec_ok = ((uintptr_t)x % 8 == 0 && model->d0 % 2 == 0) ? 1 : 0;
+  // vector loads of the rows: 8 bytes (22 -> 40) or 16 bytes (64 -> 128)
+  a.x_vec_ok = ((uintptr_t)x % (plan.wide ? 16 : 8) == 0 && model->d0 % 2 == 0) ? 1 : 0;
   a.y_vec_ok = ((uintptr_t)y % 16 == 0) ? 1 : 0;
   a.chains_per_window = 1;
   a.fixed_window = 0;
@@ -572,7 +594,7 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
   set_grid(a, 1, G, &wgs);
   // barrier and status words start from zero on every call
   HIP_TRY(launch_fill_u32(w.barrier, BARRIER_STRIDE_WORDS + 64, 0u, st));
-  HIP_TRY(launch_hmc_kernel(plan.kernel, a, wgs, plan.threads, st));
+  HIP_TRY(launch_hmc_kernel(plan.kernel, a, wgs, plan.threads, plan.dyn_lds, st));
   return BNNHMC_OK;
 }
 
@@ -702,7 +724,8 @@ int bnnhmc_create(const bnnhmc_model* model, const bnnhmc_hmc* hmc, const bnnhmc
       (rc = s->alloc(&s->tr_eps, C * s->trace_len)) || (rc = s->alloc(&ws, s->workspace_bytes)) ||
       (rc = s->alloc(&s->tmp, (size_t)3 * s->st_stride * eval_groups_max)) ||
       (rc = s->alloc(&s->tmp_ell, (size_t)s->n_pad)) ||
-      (rc = s->alloc(&s->tmp_sums, (size_t)2 * eval_groups_max)))
+      (rc = s->alloc(&s->tmp_sums, (size_t)2 * eval_groups_max)) ||
+      (rc = s->alloc(&s->wg_scratch, (size_t)s->plan.resident_wgs * s->plan.wg_scratch_floats)))
     return bail(rc);
   s->workspace = ws;
   if (getenv("BNNHMC_DEBUG_PHASE")) {

@@ -113,6 +113,7 @@ struct KArgs {
   unsigned* barrier;   // [group][BARRIER_STRIDE_WORDS]
   unsigned* status;    // [0] abort flag, [1] timed-out workgroup + 1
   unsigned spin_limit;
+  float* wg_scratch;   // wide-layer kernel, MODE_TRANSITIONS: [workgroup][3][P_AL] accepted w, g and start momentum
   int debug_drop_rank; // >= 0: this rank of every group never signals arrival (exercises the timeout path)
   unsigned* debug_xcc; // optional [workgroup] XCC id
   unsigned long long* debug_phase;  // optional [workgroup][8] cycles spent per phase of a step

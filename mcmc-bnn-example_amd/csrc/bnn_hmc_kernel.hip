@@ -1076,10 +1076,10 @@ const void* hmc_kernel_for(int d0, int d1, int layer, int lik, int threads, int 
 }
 
 hipError_t launch_hmc_kernel(const void* kernel, const KArgs& args, int workgroups, int threads,
-                             hipStream_t stream) {
+                             size_t dyn_lds_bytes, hipStream_t stream) {
   KArgs a = args;
   void* params[] = {&a};
-  return hipLaunchKernel(kernel, dim3(workgroups), dim3(threads), params, 0, stream);
+  return hipLaunchKernel(kernel, dim3(workgroups), dim3(threads), params, dyn_lds_bytes, stream);
 }
 
 }  // namespace bnn

@@ -11,8 +11,12 @@ namespace bnn {
 // trajectory kernel for (d0, d1, layer, likelihood, threads per workgroup, software-pipelined tile
 // loop or plain loop); nullptr if unsupported
 const void* hmc_kernel_for(int d0, int d1, int layer, int lik, int threads, int pipeline);
+// trajectory kernel for layers too wide for register-resident parameters (64 -> 128 -> 1); also
+// returns its dynamic LDS size and the floats of private global scratch each workgroup needs
+const void* hmc_kernel_wide_for(int d0, int d1, int lik, int threads, size_t* dyn_lds_bytes,
+                                size_t* wg_scratch_floats);
 hipError_t launch_hmc_kernel(const void* kernel, const KArgs& args, int workgroups, int threads,
-                             hipStream_t stream);
+                             size_t dyn_lds_bytes, hipStream_t stream);
 
 // small kernels
 hipError_t launch_fill_u32(unsigned* p, size_t n, unsigned v, hipStream_t stream);
