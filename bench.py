@@ -23,6 +23,8 @@ sys.path.insert(0, ROOT)
 
 N_ROWS, D0, D1 = 58368, 22, 40
 FLOP_PER_EVAL = 4 * N_ROWS * D1 * (D0 + 1)  # 214,794,240: both layers, forward + weight gradients
+# --shape wide: BASELINE.json configs[4], 64->128->1 on 4 x 58368 rows, 4 chains per window
+WIDE_ROWS, WIDE_D0, WIDE_D1, WIDE_CHAINS = 4 * 58368, 64, 128, 4
 PEAK_TFLOPS = 157.3                         # MI355X dense FP32 matrix peak (v_mfma_f32_16x16x4_f32)
 EVALS_200x800 = 200 * (900 * 1000 + 1)      # 200 windows x ((100 + 800) transitions x 1000 steps + bootstrap)
 EVALS_200x1600 = 200 * (1700 * 1000 + 1)
@@ -32,21 +34,21 @@ EVALS_200x1600 = 200 * (1700 * 1000 + 1)
 TRAFFIC_BYTES_PER_EVAL_MFMA = 8.697e11 / 160000
 
 
-def cpu_baseline(seconds):
+def cpu_baseline(seconds, n_rows=N_ROWS, d0=D0, d1=D1):
     """The CPU oracle (a port of the reference math), timed on this host's cores on one window."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import orc_binding as ob
 
     orc = ob.load()
-    X, y, _ = orc.gen_window(0, 0, N_ROWS)
-    m = ob.gauss_model(n=N_ROWS)
+    X, y, _ = orc.gen_window(0, 0, n_rows, d0=d0, d1=d1)
+    m = ob.gauss_model(n=n_rows, d0=d0, d1=d1)
     threads = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1)
     threads = max(1, min(threads, os.cpu_count() or 1))
     rate, used, done = orc.bench_grad_evals(m, X, y, threads, seconds)
     return {"value": rate, "unit": "grad-evals/s", "cores": used, "kind": "port",
-            "sample": "%d leapfrog gradient evaluations of one 58368-row window in %.0f s, one chain per "
-                      "thread" % (done, seconds),
-            "extrapolated_minutes_200x800": EVALS_200x800 / rate / 60.0}
+            "sample": "%d leapfrog gradient evaluations of one %d-row window in %.0f s, one chain per "
+                      "thread" % (done, n_rows, seconds),
+            "extrapolated_minutes_200x800": EVALS_200x800 / rate / 60.0 if d0 == D0 else None}
 
 
 def main():
@@ -63,6 +65,9 @@ def main():
     ap.add_argument("--leapfrog", type=int, default=1000)
     ap.add_argument("--transitions-per-launch", type=int, default=5)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="0 skips the CPU baseline")
+    ap.add_argument("--shape", choices=["base", "wide"], default="base",
+                    help="base = configs[2] (22->40->1, the metric's configuration); wide = configs[4] "
+                         "(64->128->1, 233472 rows, 4 chains per window)")
     ap.add_argument("--full", action="store_true",
                     help="run the whole 200 windows x (100 + 800) transitions job and time all of it")
     args = ap.parse_args()
@@ -90,15 +95,23 @@ def main():
         launch.threads = args.threads
     if args.pipeline:
         launch.pipeline = args.pipeline
-    wgs_per_cu = launch.wgs_per_cu if layer == pkg.LAYER_MFMA else 1
+    wide = args.shape == "wide"
+    if wide and args.full:
+        print("--full is the 22->40->1 job; it is not defined for --shape wide", file=sys.stderr)
+        sys.exit(2)
+    n_rows, d0, d1, cpw = (WIDE_ROWS, WIDE_D0, WIDE_D1, WIDE_CHAINS) if wide else (N_ROWS, D0, D1, 1)
+    flop_per_eval = 4 * n_rows * d1 * (d0 + 1)
+    wgs_per_cu = 1 if wide or layer != pkg.LAYER_MFMA else launch.wgs_per_cu
     group = launch.cus_per_chain or 4
-    resident = max(1, (cus * wgs_per_cu) // group)
-    n_windows = 200 if args.full else (args.windows or resident)
+    resident = max(1, (cus * wgs_per_cu) // group)          # chains in flight
+    n_windows = 200 if args.full else (args.windows or max(1, resident // cpw))
+    n_chains = n_windows * cpw
 
-    model = lib.default_model(lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
+    model = lib.default_model(d0=d0, d1=d1, n=n_rows, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01,
+                              prior_scale=0.1)
     burn, keep = (100, 800) if args.full else (args.warmup + args.steps, 0)
     hmc = lib.default_hmc(leapfrog_steps=args.leapfrog, burn_in=burn, n_samples=keep, seed=0)
-    s = lib.create(model, hmc, launch, n_windows, 1)
+    s = lib.create(model, hmc, launch, n_windows, cpw)
     for w in range(n_windows):
         s.generate_window(w, teacher_scale=0.1, noise_sigma=0.01)  # untimed, like the reference's load
 
@@ -128,14 +141,14 @@ def main():
     st = s.get_chain_state(0)
     s.close()
 
-    evals = n_windows * steps * args.leapfrog + (n_windows if args.full else 0)
+    evals = n_chains * steps * args.leapfrog + (n_chains if args.full else 0)
     value = evals / wall
     # dominant kernel: the trajectory kernel.  Average launch duration from HIP events recorded on the
     # sampler's stream around the launches of the timed region.
     dev_ms = tm1["kernel_ms"] - tm0["kernel_ms"]
     launches = tm1["launches"] - tm0["launches"]
     ms_per_launch = dev_ms / max(1, launches)
-    flop_per_launch = FLOP_PER_EVAL * (n_windows * steps * args.leapfrog) / max(1, launches)
+    flop_per_launch = flop_per_eval * (n_chains * steps * args.leapfrog) / max(1, launches)
     achieved = flop_per_launch / (ms_per_launch * 1e-3) / 1e12
 
     out = {
@@ -152,18 +165,19 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "configs[2]: %d independent windows x 1 chain (%d resident per launch), 22->40->1 BNN, "
-                        "58368x22 features ~N(0,1), teacher-MLP targets + N(0,0.01^2), Gaussian likelihood and "
-                        "prior, %d leapfrog steps per transition" % (n_windows, min(n_windows, resident),
-                                                                    args.leapfrog),
+            "workload": "configs[%d]: %d independent windows x %d chain(s) (%d chains resident per launch), "
+                        "%d->%d->1 BNN, %dx%d features ~N(0,1), teacher-MLP targets + N(0,0.01^2), Gaussian "
+                        "likelihood and prior, %d leapfrog steps per transition" % (
+                            4 if wide else 2, n_windows, cpw, min(n_chains, resident), d0, d1, n_rows, d0,
+                            args.leapfrog),
             "layer": args.layer, "cus_per_chain": group, "wgs_per_cu": wgs_per_cu,
             "workgroups": tm1["workgroups"], "compute_units": cus,
             "transitions_per_launch": args.transitions_per_launch,
         },
-        "minutes_200x800": EVALS_200x800 / value / 60.0,
-        "minutes_200x800_kind": "measured: the whole job was run" if args.full
-                                else "extrapolated from the timed transitions",
-        "minutes_200x1600_extrapolated": EVALS_200x1600 / value / 60.0,
+        "minutes_200x800": None if wide else EVALS_200x800 / value / 60.0,
+        "minutes_200x800_kind": "not defined for this shape" if wide else (
+            "measured: the whole job was run" if args.full else "extrapolated from the timed transitions"),
+        "minutes_200x1600_extrapolated": None if wide else EVALS_200x1600 / value / 60.0,
         "reference_minutes_200x800_1xA100_tf32": 42,
         "accept_rate_chain0": st["n_accepted"] / max(1, st["transitions_done"]),
         "eps_chain0": st["eps"],
@@ -171,14 +185,14 @@ def main():
             "bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": achieved / PEAK_TFLOPS,
             "traffic": (TRAFFIC_BYTES_PER_EVAL_MFMA * n_windows * steps * args.leapfrog / max(1, launches)
-                        if args.layer == "mfma" else None),
+                        if args.layer == "mfma" and not wide else None),
             "traffic_unit": "bytes per launch (measured offline with rocprofv3 --pmc, see profiles/)",
-            "kernel": "hmc_kernel", "launches": launches, "ms_per_launch": ms_per_launch,
-            "flop_per_grad_eval": FLOP_PER_EVAL,
+            "kernel": "hmc_kernel_wide" if wide else "hmc_kernel", "launches": launches,
+            "ms_per_launch": ms_per_launch, "flop_per_grad_eval": flop_per_eval,
         },
     }
     if args.cpu_seconds > 0:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
+        out["cpu_baseline"] = cpu_baseline(args.cpu_seconds, n_rows, d0, d1)
     print(json.dumps(out))
 
 
