@@ -94,7 +94,8 @@ int bnnhmc_device_info(int* n_devices, int* compute_units, char* arch, size_t ar
 
 /* Device scratch the step operator needs (per-workgroup gradient partials and barrier words); the
  * counterpart of the reference's grid_sync_workspace (include/mcmc/main.h:171,
- * include/mcmc/mcmc_step_tc.h:597-612). */
+ * include/mcmc/mcmc_step_tc.h:597-612).  The workspace must be 16-byte aligned (any hipMalloc
+ * result is). */
 size_t bnnhmc_step_workspace_bytes(const bnnhmc_model* model, const bnnhmc_launch* launch);
 
 /* L fused leapfrog steps.  Replaces mcmc::mcmc_step<T, LP_STEPS>

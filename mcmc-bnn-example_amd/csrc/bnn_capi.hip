@@ -542,6 +542,8 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
       !grad_cur || !loss_values || !workspace)
     return fail(BNNHMC_ERR_INVALID, "null device pointer passed to bnnhmc_mcmc_step");
   if (lp_steps < 1) return fail(BNNHMC_ERR_INVALID, "lp_steps must be >= 1, got %d", lp_steps);
+  if ((uintptr_t)workspace % 16 != 0)
+    return fail(BNNHMC_ERR_INVALID, "workspace must be 16-byte aligned");
   DeviceInfo di;
   rc = query_device(di);
   if (rc) return rc;

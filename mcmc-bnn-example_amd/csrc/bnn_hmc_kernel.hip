@@ -658,7 +658,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   constexpr int PPT = (P + T - 1) / T;
 
   __shared__ float s_w[P_AL];
-  __shared__ float s_slots[W][SLOT];
+  __shared__ __align__(16) float s_slots[W][SLOT];
   __shared__ double s_red[W];
   __shared__ int s_flag;
 
@@ -827,25 +827,43 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       BNN_PHASE(5)  // group barrier
       const float* grp_part = part_base + (size_t)buf * a.G * SLOT;
       if (!a.two_phase) {
-        // ---- stage 2 (small groups): every workgroup adds the G records in rank order; the prior
-        //      gradient seeds the sum as block 0 does in the reference (mcmc_step_ffma.h:144) ----
-#pragma unroll
-        for (int i = 0; i < PPT; ++i) {
-          const int p = tid + i * T;
-          if (p < P) {
-            float v = prior_grad(mc, w[i]);
-            // eight loads in flight at a time; the additions keep the order r = 0, 1, 2, ...
-            for (int r0 = 0; r0 < a.G; r0 += 8) {
-              float t8[8];
+        // ---- stage 2 (small groups): every workgroup adds the G records.  A thread takes one 16-byte
+        //      column of the records and every H-th record (H = T / 256 thread sets), eight loads in
+        //      flight, records in ascending order; the sets are then added in a fixed order through
+        //      LDS, seeded with the prior gradient as block 0 does in the reference
+        //      (mcmc_step_ffma.h:144) ----
+        constexpr int NCOL = P_AL / 4, CW = 256, H = T / CW;
+        static_assert(NCOL <= CW && T % CW == 0 && H <= W, "stage 2 thread sets");
+        {
+          const int col = tid & (CW - 1), part = tid / CW;  // part is uniform within a wave
+          if (col < NCOL) {
+            f4 v = {0.f, 0.f, 0.f, 0.f};
+            const float* src = grp_part + 4 * col;
+            for (int r0 = part; r0 < a.G; r0 += 8 * H) {
+              f4 t8[8];
 #pragma unroll
               for (int k = 0; k < 8; ++k) {
-                const int r = r0 + k < a.G ? r0 + k : a.G - 1;
-                t8[k] = ld_agent(grp_part + (size_t)r * SLOT + p);
+                const int r = r0 + H * k;
+                if (r < a.G) ld_agent4_issue(t8[k], src + (size_t)r * SLOT);
+                else t8[k] = f4{0.f, 0.f, 0.f, 0.f};
               }
+              wait_agent4x8(t8);
 #pragma unroll
-              for (int k = 0; k < 8; ++k) v += r0 + k < a.G ? t8[k] : 0.0f;
+              for (int k = 0; k < 8; ++k) v += t8[k];
             }
-            g[i] = v;
+            // rows 0 .. H-1 of s_slots are free: stage 1 read them before the barrier
+            *reinterpret_cast<f4*>(&s_slots[part][4 * col]) = v;
+          }
+          __syncthreads();
+#pragma unroll
+          for (int i = 0; i < PPT; ++i) {
+            const int p = tid + i * T;
+            if (p < P) {
+              float v = prior_grad(mc, w[i]);
+#pragma unroll
+              for (int h = 0; h < H; ++h) v += s_slots[h][p];
+              g[i] = v;
+            }
           }
         }
         if (last) {

@@ -415,20 +415,28 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
       // ---- stage 2: every workgroup adds the G records in rank order, seeded with the prior
       //      gradient (mcmc_step_ffma.h:144) ----
       const float* grp_part = part_base + (size_t)buf * a.G * SLOT;
-      for (int p = tid; p < P; p += T) {
-        float v = prior_grad(mc, s_w[p]);
+      // a thread takes 16-byte columns of the records, eight loads in flight, records in rank order
+      for (int col = tid; col < P_AL / 4; col += T) {
+        f4 v = {0.f, 0.f, 0.f, 0.f};
+        const float* src = grp_part + 4 * col;
         for (int r0 = 0; r0 < a.G; r0 += 8) {
-          float t8[8];
+          f4 t8[8];
 #pragma unroll
           for (int k = 0; k < 8; ++k) {
-            const int r = r0 + k < a.G ? r0 + k : a.G - 1;
-            t8[k] = ld_agent(grp_part + (size_t)r * SLOT + p);
+            if (r0 + k < a.G) ld_agent4_issue(t8[k], src + (size_t)(r0 + k) * SLOT);
+            else t8[k] = f4{0.f, 0.f, 0.f, 0.f};
           }
+          wait_agent4x8(t8);
 #pragma unroll
-          for (int k = 0; k < 8; ++k) v += r0 + k < a.G ? t8[k] : 0.0f;
+          for (int k = 0; k < 8; ++k) v += t8[k];
         }
-        s_g[p] = v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int p = 4 * col + e;
+          if (p < P) s_g[p] = prior_grad(mc, s_w[p]) + v[e];
+        }
       }
+      __syncthreads();  // the columns are not the parameters a thread owns in the update loops
       if (last) {
         double d = 0.0;
         for (int r = 0; r < a.G; ++r) {

@@ -89,6 +89,18 @@ __device__ __forceinline__ float ld_agent(const float* p) {
 __device__ __forceinline__ void st_agent(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// 16-byte agent-scope load, issued without waiting: up to eight of them are collected with
+// wait_agent4x8 (the compiler neither reorders nor waits for loads issued from inline assembly)
+__device__ __forceinline__ void ld_agent4_issue(f4& d, const float* p) {
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(d) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void wait_agent4x8(f4 (&t)[8]) {
+  asm volatile("s_waitcnt vmcnt(0)"
+               : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]),
+                 "+v"(t[7])
+               :
+               : "memory");
+}
 
 // ------------------------------------------------------------------------------------------------
 // Per-wave working set handed to a layer for one leapfrog step
@@ -107,17 +119,26 @@ struct StepCtx {
 // group barrier: all G workgroups of a chain group have published their partials of this step.
 // Bounded: after spin_limit polls, or when another workgroup has given up, the wait ends and the
 // launch is abandoned (status[0] set), so every wave always exits.
+//
+// Everything the workgroups of a group exchange is written with st_agent (write-through to the point
+// where all XCDs see it) and read with ld_agent / ld_agent4 (never served from an XCD-local cache
+// level), so the barrier needs no L2 write-back and no cache invalidate -- each costs microseconds
+// per step and an invalidate would also throw away the cached rows of X.  What it does need is
+// ordering: every thread waits until its own stores have been acknowledged (s_waitcnt vmcnt(0))
+// before the workgroup signals its arrival, and the exchange loads are issued after the wait.
+// Data that is not written with st_agent (per-row log-likelihood terms, chain state, samples) is only
+// ever read back by the workgroup that wrote it or after the kernel has ended.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ bool group_barrier(unsigned* counter, unsigned target, unsigned* status,
                                               unsigned spin_limit, int* s_flag, bool signal = true) {
-  __syncthreads();  // this workgroup's partials are stored (and waited for)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partials have reached memory
+  __syncthreads();
   if (threadIdx.x == 0) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     if (signal) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     unsigned polls = 0;
     int ok = 1;
     while ((int)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
-      __builtin_amdgcn_s_sleep(2);
+      __builtin_amdgcn_s_sleep(1);
       if ((++polls & 63u) == 0u) {
         if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
           ok = 0;
@@ -132,7 +153,6 @@ __device__ __forceinline__ bool group_barrier(unsigned* counter, unsigned target
         }
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     *s_flag = ok;
   }
   __syncthreads();
