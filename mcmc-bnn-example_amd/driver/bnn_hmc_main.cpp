@@ -4,7 +4,7 @@
 //
 //   bnn_hmc_main [--windows W] [--chains C] [--samples S] [--burn-in B] [--leapfrog L] [--rows N]
 //                [--lik student_t|gaussian] [--layer mfma|ffma] [--cus-per-chain G] [--wgs-per-cu K]
-//                [--seed S] [--data FILE] [--dump FILE]
+//                [--seed S] [--data FILE] [--dump FILE] [--features D0 --hidden D1]   (22 40 or 64 128)
 //
 // Without --data every window is filled with the synthetic recipe (features ~ N(0,1), targets from
 // a random teacher MLP plus noise).  With --data the reference's text format is read
@@ -23,6 +23,7 @@ namespace {
 
 struct Options {
   int windows = 1, chains = 1, samples = 800, burn_in = 100, leapfrog = 1000, rows = 58368;
+  int features = 22, hidden = 40;
   int lik = BNNHMC_LIK_STUDENT_T, layer = BNNHMC_LAYER_MFMA, cus_per_chain = 0, wgs_per_cu = 0;
   unsigned seed = 0;
   std::string data, dump;
@@ -47,6 +48,8 @@ bool parse(int argc, char** argv, Options& o) {
     else if (a == "--burn-in") o.burn_in = std::atoi(next());
     else if (a == "--leapfrog") o.leapfrog = std::atoi(next());
     else if (a == "--rows") o.rows = std::atoi(next());
+    else if (a == "--features") o.features = std::atoi(next());
+    else if (a == "--hidden") o.hidden = std::atoi(next());
     else if (a == "--seed") o.seed = (unsigned)std::strtoul(next(), nullptr, 10);
     else if (a == "--cus-per-chain") o.cus_per_chain = std::atoi(next());
     else if (a == "--wgs-per-cu") o.wgs_per_cu = std::atoi(next());
@@ -84,6 +87,8 @@ int main(int argc, char** argv) {
   bnnhmc_model model;
   bnnhmc_default_model(&model);
   model.n = o.rows;
+  model.d0 = o.features;
+  model.d1 = o.hidden;
   model.lik_kind = o.lik;
   if (o.lik == BNNHMC_LIK_GAUSSIAN) {  // the benchmark configs: sigma 0.01, prior N(0, 0.1^2)
     model.lik_scale = 0.01;
