@@ -42,10 +42,12 @@ enum KernelMode : int {
 
 // Number of floats of one workgroup's partial-result record: P gradient partials padded to a
 // multiple of 4, then 4 words of which the first two hold a double (sum of per-row log-likelihood
-// terms).
-inline int partial_slot_floats(int P) { return ((P + 3) / 4) * 4 + 4; }
+// terms); rounded up to whole 128-byte lines so that a 32-parameter slice of a record is one line.
+inline int partial_slot_floats(int P) { return (((P + 3) / 4) * 4 + 4 + 31) / 32 * 32; }
 
-constexpr int BARRIER_STRIDE_WORDS = 32;  // one 128-byte line per chain group
+// barrier words per chain group: the group's counter and eight block counters (one per 32 ranks,
+// used by groups of more than 64 workgroups), each on its own 128-byte line
+constexpr int BARRIER_STRIDE_WORDS = 32 * 9;
 
 struct KArgs {
   // ---- model / data ----

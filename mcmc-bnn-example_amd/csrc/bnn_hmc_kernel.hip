@@ -654,7 +654,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   constexpr int W = T / 64;
   constexpr int P = Layer::P;
   constexpr int P_AL = Layer::P_AL;
-  constexpr int SLOT = P_AL + 4;
+  constexpr int SLOT = (P_AL + 4 + 31) / 32 * 32;  // partial_slot_floats(P)
   constexpr int PPT = (P + T - 1) / T;
 
   __shared__ float s_w[P_AL];
@@ -696,7 +696,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   const ModelConsts mc = a.mc;
   float* part_base = a.partials + (size_t)group * 2 * a.G * SLOT;
   unsigned* counter = a.barrier + (size_t)group * BARRIER_STRIDE_WORDS;
-  unsigned bar_target = 0;
+  unsigned bar_epoch = 0;
   int buf = 0;
 
   // ---- parameters owned by this thread: p = tid + i T ----
@@ -821,8 +821,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         st_agent(my_part + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)));
       }
       BNN_PHASE(4)  // stage 1 + global store
-      bar_target += (unsigned)a.G;
-      ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag, rank != a.debug_drop_rank);
+      ok = group_barrier(counter, a.G, rank, ++bar_epoch, a.status, a.spin_limit, &s_flag, rank != a.debug_drop_rank);
       if (!ok) break;
       BNN_PHASE(5)  // group barrier
       const float* grp_part = part_base + (size_t)buf * a.G * SLOT;
@@ -877,32 +876,47 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
           dl_total = d;
         }
       } else {
-        // ---- stage 2 (large groups), in two phases.  Phase 1: workgroup `rank` reduces the slice
-        //      [rank S, rank S + S) of the parameters over all G records: 32 lanes per parameter, lane
-        //      `sub` adds records sub, sub + 32, ... in order, then a fixed xor tree over the 32 lanes.
-        //      Phase 2 (after a second group barrier): everyone reads the P totals. ----
+        // ---- stage 2 (large groups), in two phases.  Phase 1: workgroup `rank` < ceil(P / 32)
+        //      reduces the 32-parameter slice [32 rank, 32 rank + 32) -- one 128-byte line of every
+        //      record, so that no fetched line is mostly unused -- over all G records: thread
+        //      (record lane rl = tid / 8, 16-byte column c = tid % 8) adds records rl, rl + T/8, ...
+        //      in order, the record lanes of a wave are added by a fixed xor tree and the waves in
+        //      order through LDS.  Phase 2 (after a second group barrier): everyone reads the totals. ----
         float* tot = a.totals + (size_t)group * SLOT;
-        const int S = (P + a.G - 1) / a.G;
-        const int sub = tid & 31;
-        for (int base = 0; base < S; base += T / 32) {
-          const int pi = base + (tid >> 5);
-          const int p = rank * S + pi;
-          const bool act = pi < S && p < P;
-          const int pc = act ? p : 0;
-          float v = 0.0f;
-          for (int r0 = sub; r0 < a.G; r0 += 8 * 32) {
-            float t8[8];
+        constexpr int RL = T / 8;  // record lanes of a workgroup
+        if (32 * rank < P) {
+          const int c = tid & 7, rl = tid >> 3;
+          const float* src = grp_part + 32 * rank + 4 * c;
+          f4 v = {0.f, 0.f, 0.f, 0.f};
+          for (int r0 = rl; r0 < a.G; r0 += 8 * RL) {
+            f4 t8[8];
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
-              const int r = r0 + 32 * k < a.G ? r0 + 32 * k : a.G - 1;
-              t8[k] = ld_agent(grp_part + (size_t)r * SLOT + pc);
+              const int r = r0 + RL * k;
+              if (r < a.G) ld_agent4_issue(t8[k], src + (size_t)r * SLOT);
+              else t8[k] = f4{0.f, 0.f, 0.f, 0.f};
             }
+            wait_agent4x8(t8);
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v += r0 + 32 * k < a.G ? t8[k] : 0.0f;
+            for (int k = 0; k < 8; ++k) v += t8[k];
           }
 #pragma unroll
-          for (int msk = 1; msk < 32; msk <<= 1) v += __shfl_xor(v, msk);
-          if (act && sub == 0) st_agent(tot + p, v);
+          for (int e = 0; e < 4; ++e) {
+            float x = v[e];
+            x += __shfl_xor(x, 8);
+            x += __shfl_xor(x, 16);
+            x += __shfl_xor(x, 32);
+            v[e] = x;
+          }
+          // rows of s_slots are free: stage 1 read them before the barrier
+          if ((tid & 63) < 8) *reinterpret_cast<f4*>(&s_slots[wave][4 * c]) = v;
+        }
+        __syncthreads();
+        if (32 * rank < P && tid < 32 && 32 * rank + tid < P) {
+          float x = s_slots[0][tid];
+#pragma unroll
+          for (int wv = 1; wv < W; ++wv) x += s_slots[wv][tid];
+          st_agent(tot + 32 * rank + tid, x);
         }
         if (last && rank == a.G - 1 && wave == W - 1) {
           const int lane = tid & 63;
@@ -921,8 +935,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
             st_agent(tot + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)));
           }
         }
-        bar_target += (unsigned)a.G;
-        ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag, rank != a.debug_drop_rank);
+        ok = group_barrier(counter, a.G, rank, ++bar_epoch, a.status, a.spin_limit, &s_flag, rank != a.debug_drop_rank);
         if (!ok) break;
 #pragma unroll
         for (int i = 0; i < PPT; ++i) {

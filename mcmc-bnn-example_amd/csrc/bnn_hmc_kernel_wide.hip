@@ -288,7 +288,7 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
   constexpr int W = T / 64;
   constexpr int P = Layer::P;
   constexpr int P_AL = Layer::P_AL;
-  constexpr int SLOT = P_AL + 4;
+  constexpr int SLOT = (P_AL + 4 + 31) / 32 * 32;  // partial_slot_floats(P)
 
   extern __shared__ __align__(16) float s_dyn[];
   float* s_w = s_dyn;             // position of the trajectory (GEMM1 / pointwise operand)
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
   const ModelConsts mc = a.mc;
   float* part_base = a.partials + (size_t)group * 2 * a.G * SLOT;
   unsigned* counter = a.barrier + (size_t)group * BARRIER_STRIDE_WORDS;
-  unsigned bar_target = 0;
+  unsigned bar_epoch = 0;
   int buf = 0;
 
   const bool trans = a.mode == MODE_TRANSITIONS;
@@ -408,8 +408,7 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
       float* my_part = part_base + ((size_t)buf * a.G + rank) * SLOT;
       for (int p = tid; p < P_AL + 2; p += T)
         if (p < P || p >= P_AL) st_agent(my_part + p, s_red[p]);
-      bar_target += (unsigned)a.G;
-      ok = group_barrier(counter, bar_target, a.status, a.spin_limit, &s_flag,
+      ok = group_barrier(counter, a.G, rank, ++bar_epoch, a.status, a.spin_limit, &s_flag,
                          rank != a.debug_drop_rank);
       if (!ok) break;
       // ---- stage 2: every workgroup adds the G records in rank order, seeded with the prior
@@ -552,7 +551,7 @@ const void* hmc_kernel_wide_for(int d0, int d1, int lik, int threads, size_t* dy
                                 size_t* wg_scratch_floats) {
   if (d0 != 64 || d1 != 128 || threads != 256) return nullptr;
   using L = MfmaWideLayer<64, 128>;
-  if (dyn_lds_bytes) *dyn_lds_bytes = (size_t)(3 * L::P_AL + L::P_AL + 4) * sizeof(float);
+  if (dyn_lds_bytes) *dyn_lds_bytes = (size_t)(3 * L::P_AL + partial_slot_floats(L::P)) * sizeof(float);
   if (wg_scratch_floats) *wg_scratch_floats = (size_t)3 * L::P_AL;
   return lik == 0 ? reinterpret_cast<const void*>(&hmc_kernel_wide<L, 0, 256>)
                   : reinterpret_cast<const void*>(&hmc_kernel_wide<L, 1, 256>);
