@@ -68,7 +68,8 @@ typedef struct bnnhmc_launch {
   int layer;          /* BNNHMC_LAYER_MFMA (v_mfma_f32_16x16x4_f32) or BNNHMC_LAYER_FFMA          */
   int cus_per_chain;  /* workgroups that share one chain's rows; 0 = default: 4 for a sampler (64   */
                       /* chains in flight on 256 CUs; a smaller last batch is widened to fill the   */
-                      /* device, up to 64 per chain), 64 for the step operator                      */
+                      /* device, up to 256 per chain), 256 for the step operator; the              */
+                      /* 64 -> 128 -> 1 network takes at most 64                                    */
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */
   int threads;        /* threads per workgroup: 256, 512, 768 or 1024 (default 512 for MFMA,     */
                       /* 256 for FFMA)                                                           */

@@ -210,8 +210,8 @@ Workspace carve_workspace(void* base, int P, int wgs, int groups) {
 
 // Workgroups per chain for a batch of `groups` chains: the configured count, widened by powers of
 // two while the whole batch still fits the device (a last, smaller batch then uses every CU).
-int widen_group(int G, int groups, int resident_wgs) {
-  while (G * 2 * groups <= resident_wgs && G * 2 <= 64) G *= 2;
+int widen_group(int G, int groups, int resident_wgs, int cap) {
+  while (G * 2 * groups <= resident_wgs && G * 2 <= cap) G *= 2;
   return G;
 }
 
@@ -350,7 +350,7 @@ KArgs base_args(const bnnhmc_sampler* s) {
 
 int launch_and_count(bnnhmc_sampler* s, KArgs& a, int groups) {
   int wgs = 0;
-  set_grid(a, groups, s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs) : s->plan.G,
+  set_grid(a, groups, s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs, s->plan.wide ? 64 : 256) : s->plan.G,
            &wgs);
   HIP_TRY(launch_fill_u32(a.barrier, (size_t)groups * BARRIER_STRIDE_WORDS, 0u, s->stream));
   HIP_TRY(launch_hmc_kernel(s->plan.kernel, a, wgs, s->plan.threads, s->plan.dyn_lds, s->stream));
@@ -516,11 +516,11 @@ float bnnhmc_rng_log_uniform(uint32_t seed, uint32_t chain_id, uint32_t t) {
 // operator level
 // =================================================================================================
 // workgroups the step operator gives its single chain: the configured count, or by default the
-// largest power of two that is resident at once (at most 64: wider groups are barrier-bound)
-static int step_group(const bnnhmc_launch* launch, int resident_wgs) {
+// largest power of two that is resident at once (at most 256; 64 for the 64 -> 128 -> 1 kernel)
+static int step_group(const bnnhmc_launch* launch, int resident_wgs, int cap) {
   if (launch && launch->cus_per_chain > 0) return launch->cus_per_chain;
   int G = 1;
-  while (G * 2 <= resident_wgs && G * 2 <= 64) G *= 2;
+  while (G * 2 <= resident_wgs && G * 2 <= cap) G *= 2;
   return G;
 }
 
@@ -551,7 +551,7 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
   rc = make_plan(*model, launch, di, plan);
   if (rc) return rc;
   const Layout L = make_layout(model->d0, model->d1);
-  const int G = step_group(launch, plan.resident_wgs);
+  const int G = step_group(launch, plan.resident_wgs, plan.wide ? 64 : 256);
   if (G > plan.resident_wgs)
     return fail(BNNHMC_ERR_RESIDENCY, "%d workgroups per chain requested but only %d can be resident", G,
                 plan.resident_wgs);
@@ -608,7 +608,7 @@ int bnnhmc_step_check(const bnnhmc_model* model, const bnnhmc_launch* launch, vo
     DeviceInfo di;
     int rc = query_device(di);
     if (rc) return rc;
-    G = step_group(launch, di.cus);
+    G = step_group(launch, di.cus, model->d0 == 64 ? 64 : 256);
   }
   Workspace w = carve_workspace(workspace, make_layout(model->d0, model->d1).P, G, 1);
   unsigned st[2] = {0, 0};
