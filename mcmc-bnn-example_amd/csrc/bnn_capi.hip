@@ -731,7 +731,7 @@ int bnnhmc_create(const bnnhmc_model* model, const bnnhmc_hmc* hmc, const bnnhmc
     return bail(rc);
   s->workspace = ws;
   if (getenv("BNNHMC_DEBUG_PHASE")) {
-    if ((rc = s->alloc(&s->debug_phase, (size_t)8 * 4096))) return bail(rc);
+    if ((rc = s->alloc(&s->debug_phase, (size_t)10 * 4096))) return bail(rc);
   }
   e = hipMemsetAsync(s->y, 0, (size_t)n_windows * s->n_pad * sizeof(float), s->stream);
   if (e == hipSuccess) e = hipMemsetAsync(ws, 0, s->workspace_bytes, s->stream);
@@ -886,17 +886,20 @@ int bnnhmc_run(bnnhmc_sampler* s, int n_transitions) {
   HIP_TRY(hipEventElapsedTime(&ms, s->ev0, s->ev1));
   if (s->debug_phase) {
     // cycles per phase of the last launch, averaged over its workgroups
-    std::vector<unsigned long long> h((size_t)8 * s->last_workgroups);
+    std::vector<unsigned long long> h((size_t)10 * s->last_workgroups);
     HIP_TRY(hipMemcpy(h.data(), s->debug_phase, h.size() * sizeof(h[0]), hipMemcpyDeviceToHost));
     double tot[8] = {0};
     for (int wgi = 0; wgi < s->last_workgroups; ++wgi)
-      for (int k = 0; k < 8; ++k) tot[k] += (double)h[(size_t)wgi * 8 + k] / s->last_workgroups;
+      for (int k = 0; k < 8; ++k) tot[k] += (double)h[(size_t)wgi * 10 + k] / s->last_workgroups;
     const char* names[8] = {"update+sync", "operand fetch", "tile loop", "partials->LDS+sync",
                             "stage1+store", "group barrier", "stage2", "epilogue"};
     double sum = 0;
     for (int k = 0; k < 8; ++k) sum += tot[k];
     for (int k = 0; k < 8; ++k)
       fprintf(stderr, "[bnnhmc phase] %-20s %14.0f ticks %6.2f%%\n", names[k], tot[k], 100.0 * tot[k] / sum);
+    if (h[9] > 0)
+      fprintf(stderr, "[bnnhmc phase] shader clock during the launch: %.0f MHz (%llu ticks in %.3f ms)\n",
+              100.0 * (double)h[8] / (double)h[9], h[8], (double)h[9] * 1e-5);
   }
   s->kernel_ms += ms;
   s->launches += launches;

@@ -118,7 +118,7 @@ struct KArgs {
   float* wg_scratch;   // wide-layer kernel, MODE_TRANSITIONS: [workgroup][3][P_AL] accepted w, g and start momentum
   int debug_drop_rank; // >= 0: this rank of every group never signals arrival (exercises the timeout path)
   unsigned* debug_xcc; // optional [workgroup] XCC id
-  unsigned long long* debug_phase;  // optional [workgroup][8] cycles spent per phase of a step
+  unsigned long long* debug_phase;  // optional [workgroup][10]: cycles per phase of a step, launch ticks
 };
 
 }  // namespace bnn

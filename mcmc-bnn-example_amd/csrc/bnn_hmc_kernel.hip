@@ -741,7 +741,11 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
     ph[k] += now_ - tstamp;                                 \
     tstamp = now_;                                          \
   }
-  if (prof) tstamp = __builtin_readcyclecounter();
+  unsigned long long clk0 = 0, rt0 = 0;
+  if (prof) {
+    tstamp = clk0 = __builtin_readcyclecounter();
+    rt0 = __builtin_amdgcn_s_memrealtime();
+  }
   const int n_outer = trans ? a.n_trans : 1;
   double dl_total = 0.0;
 
@@ -1019,7 +1023,10 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   if (prof && tid == 0) {
     BNN_PHASE(7)  // transition epilogue
 #pragma unroll
-    for (int k = 0; k < 8; ++k) a.debug_phase[(size_t)blockIdx.x * 8 + k] = ph[k];
+    for (int k = 0; k < 8; ++k) a.debug_phase[(size_t)blockIdx.x * 10 + k] = ph[k];
+    // shader-clock ticks and 100 MHz real-time ticks of the whole launch: their ratio is the clock
+    a.debug_phase[(size_t)blockIdx.x * 10 + 8] = __builtin_readcyclecounter() - clk0;
+    a.debug_phase[(size_t)blockIdx.x * 10 + 9] = __builtin_amdgcn_s_memrealtime() - rt0;
   }
 #undef BNN_PHASE
   if (!ok) return;

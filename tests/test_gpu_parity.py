@@ -317,6 +317,46 @@ def test_full_size_properties(pkg, lib, orc):
     close_grad(halves[0] + halves[1] - prior_g, g_all.astype(np.float64), "additivity", rtol=3e-6)
 
 
+@pytest.mark.parametrize("G", [0, 4, 64])
+def test_full_size_trajectory_is_time_reversible(pkg, lib, orc, G):
+    """Leapfrog is time-reversible: L steps, the closing half kick, momentum negated, L steps again and
+    the closing half kick return to the start.  A size-independent property checked at the full
+    58368 rows (no oracle run needed); the two runs share no state but what the operator returns."""
+    say("reversibility G=%d" % G)
+    n, L, eps = 58368, 40, 0.01
+    model, om, gen = models(pkg, lib, "t", n)
+    launch = lib.default_launch(cus_per_chain=G)
+    X, y, th = orc.gen_window(11, 0, n, **gen)
+    rng = np.random.default_rng(5)
+    w0 = (th * 0.9).astype(np.float32)
+    m0 = rng.normal(0, 1, P).astype(np.float32)
+    dev = DevBuf.from_numpy
+    dX, dy = dev(X), dev(y)
+    wsb = lib.step_workspace_bytes(model, launch)
+    ws = DevBuf.full(wsb // 4 + 16, 0, np.int32)
+    dloss = DevBuf.full(n + P, 0.0)
+    dgn = DevBuf.full(P, 0.0)
+
+    def steps(w, m, g, n_steps, e):
+        dw, dm, dg = dev(w), dev(m), dev(g)
+        ow, om_, og = (DevBuf.full(P, np.nan) for _ in range(3))
+        lib.mcmc_step(model, launch, dX.ptr, dy.ptr, dw.ptr, ow.ptr, dm.ptr, om_.ptr, dg.ptr, og.ptr,
+                      dgn.ptr, dloss.ptr, ws.ptr, wsb, e, n_steps, 0)
+        lib.step_check(model, launch, ws.ptr, 0)
+        return ow.numpy(P), om_.numpy(P), og.numpy(P)
+
+    # gradient at the start: one step with eps = 0 leaves w alone and returns the gradient there
+    _, _, g0 = steps(w0, np.zeros(P, np.float32), np.zeros(P, np.float32), 1, 0.0)
+    w1, m1, g1 = steps(w0, m0, g0, L, eps)
+    m1_full = (m1 + np.float32(0.5 * eps) * g1).astype(np.float32)      # closing half kick
+    assert float(np.abs(w1 - w0).max()) > 1e-3                           # the trajectory went somewhere
+    w2, m2, g2 = steps(w1, -m1_full, g1, L, eps)
+    m2_full = m2 + np.float32(0.5 * eps) * g2
+    np.testing.assert_allclose(w2, w0, rtol=0, atol=2e-5 * max(1.0, float(np.abs(w0).max())))
+    np.testing.assert_allclose(-m2_full, m0, rtol=0, atol=2e-4)
+    close_grad(g2, g0.astype(np.float64), "gradient back at the start", rtol=5e-5)
+
+
 def test_residency_and_timeout_are_reported(pkg, lib, orc, monkeypatch):
     m = lib.default_model(n=64)
     with pytest.raises(pkg.BnnHmcError) as e:
