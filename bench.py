@@ -29,9 +29,9 @@ PEAK_TFLOPS = 157.3                         # MI355X dense FP32 matrix peak (v_m
 EVALS_200x800 = 200 * (900 * 1000 + 1)      # 200 windows x ((100 + 800) transitions x 1000 steps + bootstrap)
 EVALS_200x1600 = 200 * (1700 * 1000 + 1)
 # HBM-side bytes per gradient evaluation of the MFMA trajectory kernel, from rocprofv3 FETCH_SIZE and
-# WRITE_SIZE scaled by a 1 GiB copy kernel (profiles/hmc_kernel_mfma_22x40_32windows.txt): one window's
+# WRITE_SIZE scaled by a 1 GiB copy kernel (profiles/hmc_kernel_mfma_22x40_64windows.txt): one window's
 # X and y (5.37 MB) pass through L2 once per leapfrog step, plus the partial-gradient records.
-TRAFFIC_BYTES_PER_EVAL_MFMA = 8.697e11 / 160000
+TRAFFIC_BYTES_PER_EVAL_MFMA = 1.7288e12 / 320000
 
 
 def cpu_baseline(seconds, n_rows=N_ROWS, d0=D0, d1=D1):
