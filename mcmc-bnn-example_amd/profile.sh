@@ -1,7 +1,8 @@
 #!/bin/bash
-# Profiles the trajectory kernel on the benchmark workload with rocprofv3 and writes raw output under
-# gpurun_out/profile/.  Three passes, each its own run: kernel trace + stats, FETCH_SIZE, WRITE_SIZE
-# (plus the same two counters on a plain copy kernel of known size for calibration).
+# Profiles the trajectory kernel on the benchmark workload with rocprofv3 and writes the raw output
+# under the directory OUT set below.  Five passes, each its own run: kernel trace + stats, FETCH_SIZE,
+# WRITE_SIZE (plus the same two counters on a plain copy kernel of known size for calibration), SQ
+# counters, L2 counters.
 # Usage: bash mcmc-bnn-example_amd/profile.sh [extra bench.py arguments]
 set -e
 ROOT="$(cd "$(dirname "$0")/.." && pwd)"
