@@ -109,17 +109,23 @@ struct MfmaWideLayer {
       const float b = s_w[oB1 + 16 * t + n] * kExp2Scale;
       acc[t] = f4{b, b, b, b};
     }
+    // W1 operands come from LDS one k-step ahead of the MFMAs that use them (two register sets), so
+    // the matrix pipe never waits for an LDS read
     const float* wrow = s_w + (size_t)(KS * q) * D1 + n;
+    float bw[2][NT];
 #pragma unroll
-    for (int i = 0; i < KQ; ++i) {
+    for (int t = 0; t < NT; ++t) bw[0][t] = wrow[16 * t];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float a = ti.xa[i][e] * kExp2Scale;  // GEMM1 then yields the exp2 argument directly
-        const float* wk = wrow + (size_t)(4 * i + e) * D1;
+    for (int s = 0; s < KS; ++s) {
+      if (s + 1 < KS) {
+        const float* wk = wrow + (size_t)(s + 1) * D1;
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, wk[16 * t], acc[t], 0, 0, 0);
+        for (int t = 0; t < NT; ++t) bw[(s + 1) & 1][t] = wk[16 * t];
       }
+      const float a = ti.xa[s >> 2][s & 3] * kExp2Scale;  // GEMM1 then yields the exp2 argument directly
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bw[s & 1][t], acc[t], 0, 0, 0);
     }
     // tanh(x) = 2 / (1 + 2^t) - 1 (kernel_helpers.h:34-42 without the small-|x| identity branch)
     const float b2s = s_w[oB2] * mc.scale_recp;
