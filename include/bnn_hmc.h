@@ -221,6 +221,27 @@ int bnnhmc_final_loss(bnnhmc_sampler* s, int chain, double* loss1, double* loss2
 int bnnhmc_get_timing(bnnhmc_sampler* s, double* kernel_ms, long* launches, long* grad_evals,
                       int* workgroups);
 
+/* ------------------------------------------------------------------------------------------------
+ * Convergence diagnostics over the chains of one window (host arithmetic in double precision).
+ * No counterpart in the reference, which runs one chain per window and prints only the final
+ * losses (main.h:295-307); the scaled benchmark shape runs four chains per window, which is what
+ * these need.  Estimators of Gelman et al., Bayesian Data Analysis 3rd ed., section 11.4-11.5, as
+ * refined by Vehtari et al. 2021 (without rank normalisation):
+ *   every chain is split in halves (m = 2 * n_chains sequences of n = n_samples / 2 draws),
+ *   W = mean within-sequence variance, B / n = variance of the sequence means,
+ *   var+ = (n - 1) / n * W + B / n,   rhat = sqrt(var+ / W),
+ *   rho_t = 1 - (W - mean_j acov_j(t)) / var+,   ess = m n / (-1 + 2 sum_t P_t),
+ * where P_t = rho_2t + rho_2t+1 runs over Geyer's initial positive sequence, made monotone.
+ * A parameter that does not vary (W = 0) reports rhat = 1 and ess = m n.
+ * ---------------------------------------------------------------------------------------------- */
+
+/* samples[chain * chain_stride + draw * n_params + p] on the host; rhat and ess receive n_params
+ * doubles each (either may be NULL).  Needs n_chains >= 1 and n_samples >= 8.  No GPU involved. */
+int bnnhmc_split_rhat_ess(const float* samples, int n_chains, int n_samples, int n_params,
+                          size_t chain_stride, double* rhat, double* ess);
+/* The same over the kept samples of the chains of `window` of a sampler. */
+int bnnhmc_window_diagnostics(bnnhmc_sampler* s, int window, double* rhat, double* ess);
+
 #ifdef __cplusplus
 }
 #endif

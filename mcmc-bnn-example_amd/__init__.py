@@ -54,6 +54,7 @@ EXPORTS = [
     "bnnhmc_get_window_data", "bnnhmc_init_chains", "bnnhmc_run", "bnnhmc_get_samples",
     "bnnhmc_get_chain_state", "bnnhmc_get_traces", "bnnhmc_eval", "bnnhmc_final_loss",
     "bnnhmc_get_timing", "bnnhmc_read_reference_data", "bnnhmc_set_chain_state",
+    "bnnhmc_split_rhat_ess", "bnnhmc_window_diagnostics",
 ]
 
 
@@ -143,6 +144,18 @@ class Lib:
         self.check(self.c.bnnhmc_read_reference_data(path.encode(), C.c_int(n), C.c_int(d0),
                                                      C.c_int(total_cols), C.c_int(skip_cols), _fp(X), _fp(y)))
         return X, y
+
+    def split_rhat_ess(self, samples):
+        """samples[chain][draw][param] (float32, host) -> (split R-hat, effective sample size)."""
+        x = np.ascontiguousarray(samples, np.float32)
+        assert x.ndim == 3
+        nc, ns, npar = x.shape
+        rhat = np.empty(npar, np.float64)
+        ess = np.empty(npar, np.float64)
+        self.check(self.c.bnnhmc_split_rhat_ess(_fp(x), C.c_int(nc), C.c_int(ns), C.c_int(npar),
+                                                C.c_size_t(ns * npar), rhat.ctypes.data_as(C.c_void_p),
+                                                ess.ctypes.data_as(C.c_void_p)))
+        return rhat, ess
 
     def rng_word(self, seed, id_, stream, t, index):
         return self.c.bnnhmc_rng_word(seed, id_, stream, t, index)
@@ -288,6 +301,14 @@ class Sampler:
         self.lib.check(self.lib.c.bnnhmc_final_loss(self.h, C.c_int(chain), C.byref(a), C.byref(b),
                                                     C.byref(c)))
         return a.value, b.value, c.value
+
+    def diagnostics(self, window):
+        """(split R-hat, effective sample size) per parameter over the chains of a window."""
+        rhat = np.empty(self.P, np.float64)
+        ess = np.empty(self.P, np.float64)
+        self.lib.check(self.lib.c.bnnhmc_window_diagnostics(
+            self.h, window, rhat.ctypes.data_as(C.c_void_p), ess.ctypes.data_as(C.c_void_p)))
+        return rhat, ess
 
     def timing(self):
         ms, launches, evals, wgs = C.c_double(), C.c_long(), C.c_long(), C.c_int()

@@ -1057,6 +1057,89 @@ int bnnhmc_final_loss(bnnhmc_sampler* s, int chain, double* loss1, double* loss2
   return BNNHMC_OK;
 }
 
+int bnnhmc_split_rhat_ess(const float* samples, int n_chains, int n_samples, int n_params,
+                          size_t chain_stride, double* rhat, double* ess) {
+  if (!samples) return fail(BNNHMC_ERR_INVALID, "samples is null");
+  if (n_chains < 1 || n_params < 1) return fail(BNNHMC_ERR_INVALID, "need at least one chain and one parameter");
+  if (n_samples < 8) return fail(BNNHMC_ERR_INVALID, "need at least 8 draws per chain, got %d", n_samples);
+  const int n = n_samples / 2, m = 2 * n_chains;
+  std::vector<double> x((size_t)m * n), mean(m), var(m), acov_mean(n), rho(n);
+  for (int p = 0; p < n_params; ++p) {
+    // sequence 2c is the first half of chain c, 2c + 1 its last n draws
+    for (int c = 0; c < n_chains; ++c)
+      for (int h = 0; h < 2; ++h) {
+        const int first = h == 0 ? 0 : n_samples - n;
+        double* dst = x.data() + (size_t)(2 * c + h) * n;
+        for (int i = 0; i < n; ++i)
+          dst[i] = (double)samples[(size_t)c * chain_stride + (size_t)(first + i) * n_params + p];
+      }
+    double grand = 0.0, W = 0.0;
+    for (int j = 0; j < m; ++j) {
+      const double* xs = x.data() + (size_t)j * n;
+      double s1 = 0.0;
+      for (int i = 0; i < n; ++i) s1 += xs[i];
+      mean[j] = s1 / n;
+      double s2 = 0.0;
+      for (int i = 0; i < n; ++i) s2 += (xs[i] - mean[j]) * (xs[i] - mean[j]);
+      var[j] = s2 / (n - 1);
+      grand += mean[j] / m;
+      W += var[j] / m;
+    }
+    double B_over_n = 0.0;
+    for (int j = 0; j < m; ++j) B_over_n += (mean[j] - grand) * (mean[j] - grand) / (m - 1);
+    const double var_plus = (double)(n - 1) / n * W + B_over_n;
+    if (!(W > 0.0)) {
+      if (rhat) rhat[p] = 1.0;
+      if (ess) ess[p] = (double)m * n;
+      continue;
+    }
+    if (rhat) rhat[p] = std::sqrt(var_plus / W);
+    if (!ess) continue;
+    // rho_t for t = 0, 1, ... computed on demand; acov_j(t) with the 1 / (n - 1) normalisation
+    auto rho_at = [&](int t) {
+      double a = 0.0;
+      for (int j = 0; j < m; ++j) {
+        const double* xs = x.data() + (size_t)j * n;
+        double s = 0.0;
+        for (int i = 0; i + t < n; ++i) s += (xs[i] - mean[j]) * (xs[i + t] - mean[j]);
+        a += s / (n - 1) / m;
+      }
+      return 1.0 - (W - a) / var_plus;
+    };
+    // Geyer's initial positive sequence of pair sums, made monotone non-increasing
+    double tau = -1.0, prev_pair = 0.0;
+    bool have_prev = false;
+    for (int t = 0; t + 1 < n; t += 2) {
+      double pair = rho_at(t) + rho_at(t + 1);
+      if (!(pair > 0.0)) break;
+      if (have_prev && pair > prev_pair) pair = prev_pair;
+      tau += 2.0 * pair;
+      prev_pair = pair;
+      have_prev = true;
+    }
+    const double mn = (double)m * n;
+    tau = std::max(tau, 1.0 / std::log10(mn));
+    ess[p] = mn / tau;
+  }
+  return BNNHMC_OK;
+}
+
+int bnnhmc_window_diagnostics(bnnhmc_sampler* s, int window, double* rhat, double* ess) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  if (window < 0 || window >= s->n_windows)
+    return fail(BNNHMC_ERR_INVALID, "window %d out of range [0, %d)", window, s->n_windows);
+  const int stored =
+      std::max(0, std::min(s->hmc.n_samples, s->transitions_done - s->hmc.burn_in));
+  if (stored < 8)
+    return fail(BNNHMC_ERR_STATE, "window %d has %d kept samples per chain; 8 are needed", window, stored);
+  const size_t stride = (size_t)s->hmc.n_samples * s->L.P;
+  std::vector<float> host((size_t)s->cpw * stride);
+  HIP_TRY(hipMemcpyAsync(host.data(), s->samples + (size_t)window * s->cpw * stride,
+                         host.size() * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+  HIP_TRY(hipStreamSynchronize(s->stream));
+  return bnnhmc_split_rhat_ess(host.data(), s->cpw, stored, s->L.P, stride, rhat, ess);
+}
+
 int bnnhmc_get_timing(bnnhmc_sampler* s, double* kernel_ms, long* launches, long* grad_evals,
                       int* workgroups) {
   if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");

@@ -166,6 +166,18 @@ int main(int argc, char** argv) {
     CHECK(bnnhmc_final_loss(s, 0, &l1, &l2, &fl));
     std::printf("Final loss1: %g, loss2: %g, full loss: %g\n", l1, l2, fl);
   }
+  if (o.chains > 1 && hmc.n_samples >= 8) {
+    // convergence over the chains of window 0: worst split R-hat and smallest effective sample size
+    std::vector<double> rhat(P), ess(P);
+    CHECK(bnnhmc_window_diagnostics(s, 0, rhat.data(), ess.data()));
+    double worst = 0, least = 1e300;
+    for (int p = 0; p < P; ++p) {
+      if (rhat[p] > worst) worst = rhat[p];
+      if (ess[p] < least) least = ess[p];
+    }
+    std::printf("Window 0, %d chains: max split R-hat %.4f, min effective sample size %.1f of %d draws\n",
+                o.chains, worst, least, o.chains * hmc.n_samples);
+  }
   float eps = 0;
   int n_acc = 0, n_done = 0;
   CHECK(bnnhmc_get_chain_state(s, 0, nullptr, nullptr, &eps, &n_done, &n_acc));

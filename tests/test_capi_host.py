@@ -128,3 +128,73 @@ def test_reference_text_reader(lib, pkg, tmp_path):
     assert e.value.code == pkg.ERR_INVALID and "ends at row" in str(e.value)
     with pytest.raises(pkg.BnnHmcError):
         lib.read_reference_data(str(tmp_path / "missing.txt"), n)
+
+
+# ------------------------------------------------------------------------------------------------
+# convergence diagnostics (host arithmetic, no GPU)
+# ------------------------------------------------------------------------------------------------
+def _numpy_split_rhat_ess(x):
+    """The estimators of Vehtari et al. 2021 (no rank normalisation) written independently with numpy:
+    autocovariances by FFT, Geyer's initial positive sequence with the monotone correction."""
+    nc, ns, _ = x.shape
+    n = ns // 2
+    seq = np.concatenate([x[:, :n], x[:, ns - n:]], axis=0).astype(np.float64)  # order differs: harmless
+    m = seq.shape[0]
+    mean = seq.mean(axis=1)
+    var = seq.var(axis=1, ddof=1)
+    W = var.mean(axis=0)
+    var_plus = (n - 1) / n * W + mean.var(axis=0, ddof=1)
+    rhat = np.sqrt(var_plus / W)
+    ess = np.empty(x.shape[2])
+    for p in range(x.shape[2]):
+        c = seq[:, :, p] - mean[:, None, p]
+        f = np.fft.rfft(c, 2 * n, axis=1)
+        acov = np.fft.irfft(f * np.conj(f), 2 * n, axis=1)[:, :n] / (n - 1)
+        rho = 1.0 - (W[p] - acov.mean(axis=0)) / var_plus[p]
+        tau, prev = -1.0, None
+        for t in range(0, n - 1, 2):
+            pair = rho[t] + rho[t + 1]
+            if not pair > 0:
+                break
+            if prev is not None and pair > prev:
+                pair = prev
+            tau += 2 * pair
+            prev = pair
+        tau = max(tau, 1 / np.log10(m * n))
+        ess[p] = m * n / tau
+    return rhat, ess
+
+
+def test_split_rhat_and_ess(lib, pkg):
+    rng = np.random.default_rng(12)
+    C_, S, Pn = 4, 800, 6
+    phi = np.array([0.0, 0.5, 0.9, -0.5, 0.0, 0.0])
+    x = np.empty((C_, S, Pn), np.float64)
+    e = rng.normal(size=(C_, S + 200, Pn))
+    z = np.zeros((C_, Pn))
+    out = []
+    for t in range(S + 200):                      # stationary AR(1) with unit marginal variance
+        z = phi * z + np.sqrt(1 - phi ** 2) * e[:, t]
+        out.append(z.copy())
+    x[:] = np.stack(out[200:], axis=1)
+    x[:, :, 4] += np.array([0.0, 0.0, 0.0, 3.0])[:, None]     # one chain sits elsewhere
+    x[:, :, 5] = 1.25                                          # a parameter that never moves
+    xs = x.astype(np.float32)
+    rhat, ess = lib.split_rhat_ess(xs)
+    # against an independent numpy / FFT implementation of the same published estimators
+    r_np, e_np = _numpy_split_rhat_ess(xs[:, :, :5])
+    np.testing.assert_allclose(rhat[:5], r_np, rtol=1e-9)
+    np.testing.assert_allclose(ess[:5], e_np, rtol=1e-6)
+    # against what the processes fix: iid draws ~ all 3200 count, AR(1) keeps N (1 - phi) / (1 + phi)
+    N = C_ * S
+    assert 0.8 * N < ess[0] < 1.2 * N and rhat[0] < 1.01
+    assert ess[1] == pytest.approx(N / 3, rel=0.25) and rhat[1] < 1.02
+    assert ess[2] == pytest.approx(N / 19, rel=0.4) and rhat[2] < 1.1
+    assert ess[3] > 1.5 * N                                    # antithetic draws beat iid
+    assert rhat[4] > 1.5 and ess[4] < 20                       # disagreeing chains are flagged
+    assert rhat[5] == 1.0 and ess[5] == N                      # constant parameter
+    # one chain only: split halves still work
+    r1, e1 = lib.split_rhat_ess(xs[:1])
+    assert r1[0] < 1.02 and 0.6 * S < e1[0] < 1.4 * S
+    with pytest.raises(pkg.BnnHmcError):
+        lib.split_rhat_ess(xs[:, :7])

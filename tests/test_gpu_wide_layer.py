@@ -192,3 +192,23 @@ def test_windows_times_four_chains_are_independent_and_reproducible(pkg, lib, or
     ref = orc.run_chain(om, ob.Hmc(L, 2, T - 2, 2, 0.004, 0.2, 0.1, 0.01, 9, 0), X, y)
     np.testing.assert_allclose(a[0], ref["samples"], rtol=0,
                                atol=2e-4 * max(1.0, float(np.abs(ref["samples"]).max())))
+
+
+def test_window_diagnostics_use_the_four_chains(pkg, lib, orc):
+    n, L, burn, keep = 400, 5, 2, 10
+    model, om, gen = models(pkg, lib, "t_stiff", n)
+    hmc = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=0.004, seed=4)
+    s = lib.create(model, hmc, lib.default_launch(cus_per_chain=4), 2, 4)
+    for w in range(2):
+        s.generate_window(w, **gen)
+    s.init_chains(None)
+    s.run(burn + 4)
+    with pytest.raises(pkg.BnnHmcError):       # four kept samples so far: too few
+        s.diagnostics(1)
+    s.run(keep - 4)
+    rhat, ess = s.diagnostics(1)
+    chains = np.stack([s.get_samples(4 + c) for c in range(4)])
+    s.close()
+    r_host, e_host = lib.split_rhat_ess(chains)
+    assert rhat.tobytes() == r_host.tobytes() and ess.tobytes() == e_host.tobytes()
+    assert np.all(np.isfinite(rhat)) and np.all(rhat >= 0.5) and np.all(ess > 0)
