@@ -64,6 +64,9 @@ def main():
     ap.add_argument("--windows", type=int, default=0, help="0 = as many as are co-resident")
     ap.add_argument("--leapfrog", type=int, default=1000)
     ap.add_argument("--transitions-per-launch", type=int, default=5)
+    ap.add_argument("--eps0", type=float, default=2e-5,
+                    help="initial leapfrog step size of the timed transitions: about what the adaptation "
+                         "reaches on this posterior; --full starts from the reference's 0.01 and adapts")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="0 skips the CPU baseline")
     ap.add_argument("--shape", choices=["base", "wide"], default="base",
                     help="base = configs[2] (22->40->1, the metric's configuration); wide = configs[4] "
@@ -111,6 +114,8 @@ def main():
                               prior_scale=0.1)
     burn, keep = (100, 800) if args.full else (args.warmup + args.steps, 0)
     hmc = lib.default_hmc(leapfrog_steps=args.leapfrog, burn_in=burn, n_samples=keep, seed=0)
+    if not args.full:
+        hmc.eps0 = args.eps0
     s = lib.create(model, hmc, launch, n_windows, cpw)
     for w in range(n_windows):
         s.generate_window(w, teacher_scale=0.1, noise_sigma=0.01)  # untimed, like the reference's load
@@ -173,6 +178,7 @@ def main():
             "layer": args.layer, "cus_per_chain": group, "wgs_per_cu": wgs_per_cu,
             "workgroups": tm1["workgroups"], "compute_units": cus,
             "transitions_per_launch": args.transitions_per_launch,
+            "eps0": float(hmc.eps0),
         },
         "minutes_200x800": None if wide else EVALS_200x800 / value / 60.0,
         "minutes_200x800_kind": "not defined for this shape" if wide else (
