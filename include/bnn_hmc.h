@@ -76,7 +76,7 @@ typedef struct bnnhmc_launch {
   int pipeline;       /* MFMA tile loop: 0 or 2 = loads issued two tiles ahead with explicit     */
                       /* waits (default), 1 = software-pipelined GEMM/pointwise stages,          */
                       /* 3 = plain loop (default 1024 threads)                                   */
-  int transitions_per_launch; /* bound on one kernel's run time (default 8)                      */
+  int transitions_per_launch; /* bound on one kernel's run time (default 8; 1 for 64 -> 128 -> 1) */
   unsigned spin_limit; /* polls before an in-kernel wait gives up (default 1 << 22)              */
 } bnnhmc_launch;
 

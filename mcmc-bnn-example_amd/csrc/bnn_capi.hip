@@ -173,7 +173,10 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
                 resident);
   p.max_groups = resident / p.G;
   p.spin_limit = l.spin_limit;
-  p.transitions_per_launch = l.transitions_per_launch;
+  // a launch of the 64 -> 128 -> 1 network does 36 times the work per transition: one transition per
+  // launch keeps a kernel's run time in seconds unless the caller asks for more
+  p.transitions_per_launch =
+      p.wide && !(lp && lp->transitions_per_launch > 0) ? 1 : l.transitions_per_launch;
   return BNNHMC_OK;
 }
 
