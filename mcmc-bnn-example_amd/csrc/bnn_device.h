@@ -45,9 +45,10 @@ enum KernelMode : int {
 // terms); rounded up to whole 128-byte lines so that a 32-parameter slice of a record is one line.
 inline int partial_slot_floats(int P) { return (((P + 3) / 4) * 4 + 4 + 31) / 32 * 32; }
 
-// barrier words per chain group: the group's counter and eight block counters (one per 32 ranks,
-// used by groups of more than 64 workgroups), each on its own 128-byte line
-constexpr int BARRIER_STRIDE_WORDS = 32 * 9;
+// barrier words per chain group: the group's counter, eight block counters (one per 32 ranks, used by
+// groups of more than 64 workgroups) and the counters of the second barrier of the two-phase
+// reduction (arrivals, eight release lines), each on its own 128-byte line
+constexpr int BARRIER_STRIDE_WORDS = 32 * 18;
 
 struct KArgs {
   // ---- model / data ----

@@ -825,7 +825,11 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         st_agent(my_part + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)));
       }
       BNN_PHASE(4)  // stage 1 + global store
-      ok = group_barrier(counter, a.G, rank, ++bar_epoch, a.status, a.spin_limit, &s_flag, rank != a.debug_drop_rank);
+      // two-phase reduction: only the workgroups that reduce a slice need the others' records now
+      constexpr int N_RED = (P + 31) / 32;
+      const bool reducer = rank < N_RED;
+      ok = group_barrier(counter, a.G, rank, ++bar_epoch, a.status, a.spin_limit, &s_flag,
+                         rank != a.debug_drop_rank, !a.two_phase || reducer);
       if (!ok) break;
       BNN_PHASE(5)  // group barrier
       const float* grp_part = part_base + (size_t)buf * a.G * SLOT;
@@ -885,10 +889,12 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         //      record, so that no fetched line is mostly unused -- over all G records: thread
         //      (record lane rl = tid / 8, 16-byte column c = tid % 8) adds records rl, rl + T/8, ...
         //      in order, the record lanes of a wave are added by a fixed xor tree and the waves in
-        //      order through LDS.  Phase 2 (after a second group barrier): everyone reads the totals. ----
+        //      order through LDS.  Phase 2 (once all reducing workgroups have stored their slices):
+        //      everyone reads the totals.  Workgroups that reduce nothing do not wait for the first
+        //      barrier at all. ----
         float* tot = a.totals + (size_t)group * SLOT;
         constexpr int RL = T / 8;  // record lanes of a workgroup
-        if (32 * rank < P) {
+        if (reducer) {
           const int c = tid & 7, rl = tid >> 3;
           const float* src = grp_part + 32 * rank + 4 * c;
           f4 v = {0.f, 0.f, 0.f, 0.f};
@@ -916,13 +922,13 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
           if ((tid & 63) < 8) *reinterpret_cast<f4*>(&s_slots[wave][4 * c]) = v;
         }
         __syncthreads();
-        if (32 * rank < P && tid < 32 && 32 * rank + tid < P) {
+        if (reducer && tid < 32 && 32 * rank + tid < P) {
           float x = s_slots[0][tid];
 #pragma unroll
           for (int wv = 1; wv < W; ++wv) x += s_slots[wv][tid];
           st_agent(tot + 32 * rank + tid, x);
         }
-        if (last && rank == a.G - 1 && wave == W - 1) {
+        if (last && rank == N_RED - 1 && wave == W - 1) {
           const int lane = tid & 63;
           double d = 0.0;
           for (int r = lane; r < a.G; r += 64) {
@@ -939,7 +945,8 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
             st_agent(tot + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)));
           }
         }
-        ok = group_barrier(counter, a.G, rank, ++bar_epoch, a.status, a.spin_limit, &s_flag, rank != a.debug_drop_rank);
+        ok = reducer_barrier(counter, N_RED, reducer, rank, bar_epoch, a.status, a.spin_limit, &s_flag,
+                             rank != a.debug_drop_rank);
         if (!ok) break;
 #pragma unroll
         for (int i = 0; i < PPT; ++i) {

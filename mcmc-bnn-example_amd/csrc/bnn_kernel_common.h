@@ -129,12 +129,33 @@ struct StepCtx {
 // Data that is not written with st_agent (per-row log-likelihood terms, chain state, samples) is only
 // ever read back by the workgroup that wrote it or after the kernel has ended.
 // ------------------------------------------------------------------------------------------------
+// bounded poll of a counter by one thread: 1 when it has reached `target`, 0 when the launch is being
+// abandoned (another workgroup gave up, or this one has polled spin_limit times)
+__device__ __forceinline__ int poll_counter(unsigned* line, unsigned target, unsigned* status,
+                                            unsigned spin_limit) {
+  unsigned polls = 0;
+  while ((int)(__hip_atomic_load(line, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
+    __builtin_amdgcn_s_sleep(1);
+    if ((++polls & 63u) == 0u) {
+      if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return 0;
+      if (polls >= spin_limit) {
+        __hip_atomic_store(status + 1, (unsigned)blockIdx.x + 1u, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return 0;
+      }
+    }
+  }
+  return 1;
+}
+
 // `epoch` counts the barriers of this launch from 1.  Up to 64 workgroups add to the group's counter
 // directly.  Larger groups arrive in blocks of 32 ranks at a block counter and the last arriver of a
 // block adds to the group's counter: 256 same-address atomics cost 3.8 us, 32 + 8 cost 2.3 us.
+// With wait == false the workgroup only announces its arrival (it does not need the others' data).
 __device__ __forceinline__ bool group_barrier(unsigned* line, int G, int rank, unsigned epoch,
                                               unsigned* status, unsigned spin_limit, int* s_flag,
-                                              bool signal = true) {
+                                              bool signal = true, bool wait = true) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partials have reached memory
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -153,25 +174,35 @@ __device__ __forceinline__ bool group_barrier(unsigned* line, int G, int rank, u
           __hip_atomic_fetch_add(line, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    unsigned polls = 0;
-    int ok = 1;
-    while ((int)(__hip_atomic_load(line, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
-      __builtin_amdgcn_s_sleep(1);
-      if ((++polls & 63u) == 0u) {
-        if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
-          ok = 0;
-          break;
-        }
-        if (polls >= spin_limit) {
-          __hip_atomic_store(status + 1, (unsigned)blockIdx.x + 1u, __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_AGENT);
-          __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          ok = 0;
-          break;
-        }
+    *s_flag = wait ? poll_counter(line, target, status, spin_limit) : 1;
+  }
+  __syncthreads();
+  return *s_flag != 0;
+}
+
+// Second barrier of the two-phase reduction: only the `n_red` reducing workgroups have something to
+// announce (their slice of the totals is stored); everybody waits for all of them.  Uses the last
+// nine counter lines of the group.
+__device__ __forceinline__ bool reducer_barrier(unsigned* line, int n_red, bool reducer, int rank,
+                                                unsigned epoch, unsigned* status, unsigned spin_limit,
+                                                int* s_flag, bool signal = true) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    // the reducers count themselves on a line nobody polls; the last one releases everybody through
+    // eight polled lines (one per block of 32 ranks), each of which sees one atomic per step and 32
+    // pollers: polls of one line are served one after the other
+    unsigned* arrivals = line + 32 * 9;
+    unsigned* release = line + 32 * 10;
+    if (reducer && signal) {
+      const unsigned prev = __hip_atomic_fetch_add(arrivals, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (prev + 1u == epoch * (unsigned)n_red) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          __hip_atomic_fetch_add(release + 32 * k, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    *s_flag = ok;
+    *s_flag = poll_counter(release + 32 * ((rank >> 5) & 7), epoch, status, spin_limit);
   }
   __syncthreads();
   return *s_flag != 0;
