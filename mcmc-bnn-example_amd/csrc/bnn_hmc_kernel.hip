@@ -348,6 +348,10 @@ struct MfmaLayer {
   static __device__ __forceinline__ void gload4(f4& d, const float* p) {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
   }
+  template <int BYTES>
+  static __device__ __forceinline__ void gload2_at(f2& d, const float* p) {
+    asm volatile("global_load_dwordx2 %0, %1, off offset:%2" : "=v"(d) : "v"(p), "n"(BYTES) : "memory");
+  }
   template <int N>
   static __device__ __forceinline__ void wait_tile(TileRaw& t) {
     asm volatile("s_waitcnt vmcnt(%[cnt])"
@@ -372,15 +376,28 @@ struct MfmaLayer {
                                : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 2 * n;
     const unsigned sb = b_const ? 0u : (unsigned)tile_floats;
     const float* py = cx.y + 4 * q;
-    auto issue = [&](TileRaw& t, int tile) {  // exactly 7 loads
-      tile = tile < te ? tile : te - 1;
-      const unsigned rel = (unsigned)(tile - tb);
-      gload4(t.xa01, pa + (size_t)tile * tile_floats);
-      gload2(t.xa2, pa_last0 + (size_t)rel * sa_last);
-      const float* rb = pb0 + (size_t)rel * sb;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) gload2(t.xb[j], rb + j * D0);
-      gload4(t.yv, py + (size_t)tile * 16);
+    // running addresses of the next tile to load: the tiles are issued in order, one call each, and
+    // past the last tile the addresses stay where they are (a harmless repeated load)
+    const float* ca = pa + (size_t)tb * tile_floats;
+    const float* cl = pa_last0;
+    const float* cb = pb0;
+    const float* cy = py + (size_t)tb * 16;
+    int nxt = tb;
+    auto issue = [&](TileRaw& t, int) {  // exactly 7 loads
+      gload4(t.xa01, ca);
+      gload2(t.xa2, cl);
+      gload2_at<0>(t.xb[0], cb);
+      gload2_at<D0 * 4>(t.xb[1], cb);
+      gload2_at<2 * D0 * 4>(t.xb[2], cb);
+      gload2_at<3 * D0 * 4>(t.xb[3], cb);
+      gload4(t.yv, cy);
+      ++nxt;
+      if (nxt < te) {
+        ca += tile_floats;
+        cl += sa_last;
+        cb += sb;
+        cy += 16;
+      }
     };
     auto compute = [&](TileRaw& t, int tile) {
       wait_tile<14>(t);
