@@ -365,39 +365,54 @@ struct MfmaLayer {
   __device__ __forceinline__ void prefetch_loop(const StepCtx& cx, const ModelConsts& mc, int tb,
                                                 int te, int n, int q) {
     static_assert(KP == 3, "register sets are laid out for three k-pairs");
-    const AugTable<D0>* aug = aug_table<D0>();
-    const size_t tile_floats = (size_t)16 * D0;
-    const float* pa = cx.X + (size_t)n * D0 + KS * q;
+    // Every load is  base (wave-uniform, in SGPRs, advanced by scalar instructions)  +  a 32-bit
+    // per-lane offset that never changes: no vector instruction is spent on addresses.  Lanes whose
+    // operand slot is the constant-one feature or padding do not load at all: their registers are
+    // set once, below, and the loads of those slots run with these lanes masked out of EXEC.
+    const unsigned oa = (unsigned)((n * D0 + KS * q) * 4);
+    const unsigned ol = oa + 2 * (KP - 1) * 4;
+    const unsigned ob = (unsigned)(((4 * q) * D0 + 2 * n) * 4);
+    const unsigned oy = (unsigned)(4 * q * 4);
     const bool a_const = KS * q + 2 * (KP - 1) >= D0;
-    const float* pa_last0 = a_const ? aug->one : pa + (size_t)tb * tile_floats + 2 * (KP - 1);
-    const unsigned sa_last = a_const ? 0u : (unsigned)tile_floats;
     const bool b_const = 2 * n >= D0;
-    const float* pb0 = b_const ? (2 * n == D0 ? aug->one : aug->zero)
-                               : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 2 * n;
-    const unsigned sb = b_const ? 0u : (unsigned)tile_floats;
-    const float* py = cx.y + 4 * q;
-    // running addresses of the next tile to load: the tiles are issued in order, one call each, and
-    // past the last tile the addresses stay where they are (a harmless repeated load)
-    const float* ca = pa + (size_t)tb * tile_floats;
-    const float* cl = pa_last0;
-    const float* cb = pb0;
-    const float* cy = py + (size_t)tb * 16;
-    int nxt = tb;
+    const unsigned long long mask_a = __builtin_amdgcn_ballot_w64(!a_const);
+    const unsigned long long mask_b = __builtin_amdgcn_ballot_w64(!b_const);
+    const f2 const_a = f2{1.0f, 0.0f};
+    const f2 const_b = f2{2 * n == D0 ? 1.0f : 0.0f, 0.0f};
+    int nxt = tb;  // tiles are issued in order, one call each; past the last tile the base stays
     auto issue = [&](TileRaw& t, int) {  // exactly 7 loads
-      gload4(t.xa01, ca);
-      gload2(t.xa2, cl);
-      gload2_at<0>(t.xb[0], cb);
-      gload2_at<D0 * 4>(t.xb[1], cb);
-      gload2_at<2 * D0 * 4>(t.xb[2], cb);
-      gload2_at<3 * D0 * 4>(t.xb[3], cb);
-      gload4(t.yv, cy);
+      const int tile = nxt < te ? nxt : te - 1;
       ++nxt;
-      if (nxt < te) {
-        ca += tile_floats;
-        cl += sa_last;
-        cb += sb;
-        cy += 16;
-      }
+      const float* bx = cx.X + (size_t)tile * (16 * D0);
+      const float* by = cx.y + (size_t)tile * 16;
+      // One block for the seven loads.  The leading s_nop gives the five wait states a memory
+      // instruction needs after a VALU instruction wrote one of its SGPR operands (the compiler
+      // reloads spilled SGPRs with v_readlane and does not see the loads inside the assembly, so it
+      // would not insert them itself).  The pure outputs are early-clobber: a returning load must
+      // not land in a register that still holds an offset of a load not yet issued.
+      asm volatile(
+          "s_nop 4\n\t"
+          "global_load_dwordx4 %[xa01], %[oa], %[bx]\n\t"
+          "s_mov_b64 exec, %[ma]\n\t"
+          "global_load_dwordx2 %[xa2], %[ol], %[bx]\n\t"
+          "s_mov_b64 exec, %[mb]\n\t"
+          "global_load_dwordx2 %[xb0], %[ob], %[bx]\n\t"
+          "global_load_dwordx2 %[xb1], %[ob], %[bx] offset:%[r1]\n\t"
+          "global_load_dwordx2 %[xb2], %[ob], %[bx] offset:%[r2]\n\t"
+          "global_load_dwordx2 %[xb3], %[ob], %[bx] offset:%[r3]\n\t"
+          "s_mov_b64 exec, -1\n\t"
+          "global_load_dwordx4 %[yv], %[oy], %[by]"
+          : [xa01] "=&v"(t.xa01), [xa2] "+v"(t.xa2), [xb0] "+v"(t.xb[0]), [xb1] "+v"(t.xb[1]),
+            [xb2] "+v"(t.xb[2]), [xb3] "+v"(t.xb[3]), [yv] "=&v"(t.yv)
+          : [oa] "v"(oa), [ol] "v"(ol), [ob] "v"(ob), [oy] "v"(oy), [bx] "s"(bx), [by] "s"(by),
+            [ma] "s"(mask_a), [mb] "s"(mask_b), [r1] "n"(D0 * 4), [r2] "n"(2 * D0 * 4),
+            [r3] "n"(3 * D0 * 4)
+          : "memory");
+    };
+    auto preset = [&](TileRaw& t) {
+      t.xa2 = const_a;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t.xb[j] = const_b;
     };
     auto compute = [&](TileRaw& t, int tile) {
       wait_tile<14>(t);
@@ -408,6 +423,9 @@ struct MfmaLayer {
       gemm2(acc, t.xb);
     };
     TileRaw A, B, C;
+    preset(A);
+    preset(B);
+    preset(C);
     issue(A, tb);
     issue(B, tb + 1);
     for (int i = tb; i < te; i += 3) {
