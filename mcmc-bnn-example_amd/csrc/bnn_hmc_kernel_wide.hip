@@ -204,22 +204,40 @@ struct MfmaWideLayer {
     if (fast_end > tb) {
       // loads issued one tile ahead by inline assembly (the compiler neither moves nor waits for
       // them); s_waitcnt vmcnt(N_LOADS) leaves the newer tile in flight
-      const size_t tile_floats = (size_t)16 * D0;
-      const float* pa = cx.X + (size_t)n * D0 + KS * q;
-      const float* pb = cx.X + (size_t)(4 * q) * D0 + 2 * n;
-      const float* py = cx.y + 4 * q;
+      // every load is a wave-uniform base (SGPRs, scalar arithmetic) plus a fixed 32-bit per-lane
+      // offset plus an immediate: no vector instruction is spent on addresses.  One assembly block
+      // per tile; its leading s_nop gives the wait states a memory instruction needs after a VALU
+      // instruction (a v_readlane reloading a spilled SGPR) wrote one of its SGPR operands -- the
+      // compiler does not see the loads inside the block.  Outputs are early-clobber.
+      static_assert(KQ == 4 && FV == 2, "operand list below is written for D0 = 64");
+      const unsigned oa = (unsigned)((n * D0 + KS * q) * 4);
+      const unsigned ob = (unsigned)(((4 * q) * D0 + 2 * n) * 4);
+      const unsigned oy = (unsigned)(4 * q * 4);
       auto issue = [&](Tile& t, int tile) {
         tile = tile < fast_end ? tile : fast_end - 1;
-        const float* ra = pa + (size_t)tile * tile_floats;
-#pragma unroll
-        for (int i = 0; i < KQ; ++i) gload4(t.xa[i], ra + 4 * i);
-        const float* rb = pb + (size_t)tile * tile_floats;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-#pragma unroll
-          for (int v = 0; v < FV; ++v) gload2(t.xb[j][v], rb + j * D0 + 32 * v);
-        }
-        gload4(t.yv, py + (size_t)tile * 16);
+        const float* bx = cx.X + (size_t)tile * (16 * D0);
+        const float* by = cx.y + (size_t)tile * 16;
+        asm volatile(
+            "s_nop 4\n\t"
+            "global_load_dwordx4 %[a0], %[oa], %[bx]\n\t"
+            "global_load_dwordx4 %[a1], %[oa], %[bx] offset:16\n\t"
+            "global_load_dwordx4 %[a2], %[oa], %[bx] offset:32\n\t"
+            "global_load_dwordx4 %[a3], %[oa], %[bx] offset:48\n\t"
+            "global_load_dwordx2 %[b00], %[ob], %[bx]\n\t"
+            "global_load_dwordx2 %[b01], %[ob], %[bx] offset:128\n\t"
+            "global_load_dwordx2 %[b10], %[ob], %[bx] offset:256\n\t"
+            "global_load_dwordx2 %[b11], %[ob], %[bx] offset:384\n\t"
+            "global_load_dwordx2 %[b20], %[ob], %[bx] offset:512\n\t"
+            "global_load_dwordx2 %[b21], %[ob], %[bx] offset:640\n\t"
+            "global_load_dwordx2 %[b30], %[ob], %[bx] offset:768\n\t"
+            "global_load_dwordx2 %[b31], %[ob], %[bx] offset:896\n\t"
+            "global_load_dwordx4 %[yv], %[oy], %[by]"
+            : [a0] "=&v"(t.xa[0]), [a1] "=&v"(t.xa[1]), [a2] "=&v"(t.xa[2]), [a3] "=&v"(t.xa[3]),
+              [b00] "=&v"(t.xb[0][0]), [b01] "=&v"(t.xb[0][1]), [b10] "=&v"(t.xb[1][0]),
+              [b11] "=&v"(t.xb[1][1]), [b20] "=&v"(t.xb[2][0]), [b21] "=&v"(t.xb[2][1]),
+              [b30] "=&v"(t.xb[3][0]), [b31] "=&v"(t.xb[3][1]), [yv] "=&v"(t.yv)
+            : [oa] "v"(oa), [ob] "v"(ob), [oy] "v"(oy), [bx] "s"(bx), [by] "s"(by)
+            : "memory");
       };
       Tile A, B;
       issue(A, tb);
