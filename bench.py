@@ -31,7 +31,7 @@ EVALS_200x1600 = 200 * (1700 * 1000 + 1)
 # HBM-side bytes per gradient evaluation of the MFMA trajectory kernel, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE scaled by a 1 GiB copy kernel (profiles/hmc_kernel_mfma_22x40_64windows.txt): one window's
 # X and y (5.37 MB) pass through L2 once per leapfrog step, plus the partial-gradient records.
-TRAFFIC_BYTES_PER_EVAL_MFMA = 1.7288e12 / 320000
+TRAFFIC_BYTES_PER_EVAL_MFMA = 1.7287e12 / 320000
 
 
 def cpu_baseline(seconds, n_rows=N_ROWS, d0=D0, d1=D1):
