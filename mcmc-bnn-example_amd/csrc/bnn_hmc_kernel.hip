@@ -342,16 +342,6 @@ struct MfmaLayer {
     f2 xb[4];  // GEMM2 operand
     f4 yv;
   };
-  static __device__ __forceinline__ void gload2(f2& d, const float* p) {
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
-  }
-  static __device__ __forceinline__ void gload4(f4& d, const float* p) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
-  }
-  template <int BYTES>
-  static __device__ __forceinline__ void gload2_at(f2& d, const float* p) {
-    asm volatile("global_load_dwordx2 %0, %1, off offset:%2" : "=v"(d) : "v"(p), "n"(BYTES) : "memory");
-  }
   template <int N>
   static __device__ __forceinline__ void wait_tile(TileRaw& t) {
     asm volatile("s_waitcnt vmcnt(%[cnt])"

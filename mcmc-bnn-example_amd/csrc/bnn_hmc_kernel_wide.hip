@@ -80,12 +80,6 @@ struct MfmaWideLayer {
     }
   }
 
-  static __device__ __forceinline__ void gload2(f2& d, const float* p) {
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
-  }
-  static __device__ __forceinline__ void gload4(f4& d, const float* p) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
-  }
   // wait until at most N memory operations are outstanding; the tile's registers are tied to the
   // wait so that nothing that uses them is scheduled above it
   template <int N>
