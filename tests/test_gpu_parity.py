@@ -90,6 +90,25 @@ def test_eval_matches_oracle(pkg, lib, orc, layer, kind, n, G):
     s.close()
 
 
+@pytest.mark.parametrize("pipeline,threads", [(1, 512), (3, 512), (3, 1024), (2, 1024)])
+def test_alternative_tile_loops_match_oracle(pkg, lib, orc, pipeline, threads):
+    """The software-pipelined (1) and plain (3) tile loops and other workgroup sizes stay selectable
+    through the launch parameters; they must give the same gradients as the default loop."""
+    say("tile loop %d, %d threads" % (pipeline, threads))
+    n = 4101
+    model, om, gen = models(pkg, lib, "gauss", n)
+    s = lib.create(model, lib.default_hmc(seed=2), lib.default_launch(cus_per_chain=4, pipeline=pipeline,
+                                                                      threads=threads), 1, 1)
+    th = s.generate_window(0, **gen)
+    X, y = s.get_window_data(0)
+    w = (th * 0.6).astype(np.float32)
+    ell, prior, grad = s.eval(0, w)
+    s.close()
+    ell_o, prior_o, grad_o, _ = orc.eval_f32(om, X, y, w)
+    close_grad(grad, grad_o, "grad vs f32 oracle")
+    np.testing.assert_allclose(ell, ell_o, rtol=RTOL, atol=RTOL * max(1.0, float(np.abs(ell_o).max())))
+
+
 def test_eval_is_deterministic_and_layout_agnostic(pkg, lib, orc):
     n = 5000
     model, om, gen = models(pkg, lib, "t", n)
