@@ -9,7 +9,7 @@
 typedef float f4 __attribute__((ext_vector_type(4)));
 // 512 threads = 8 waves; wave w sits on SIMD w % 4.  role(wave) decides what the wave does.
 // ROLE: 0 all MFMA; 1 all FMA; 2 waves 0-3 MFMA, waves 4-7 FMA (one of each per SIMD); 3 all EXP (trans); 4: waves 0-3 FMA, 4-7 EXP
-// 5: waves 0-3 MFMA, 4-7 idle; 6: waves 0-3 FMA, 4-7 idle ; 7: waves 0-3 EXP, 4-7 idle
+// 5: waves 0-3 MFMA, 4-7 idle; 6: waves 0-3 FMA, 4-7 idle ; 7: waves 0-3 EXP, 4-7 idle; 8: waves 0-3 MFMA, 4-7 EXP
 template <int ROLE>
 __global__ __launch_bounds__(512) void k(float* out, int iters, float a, float b) {
   int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -17,7 +17,7 @@ __global__ __launch_bounds__(512) void k(float* out, int iters, float a, float b
   int what; // 0 mfma 1 fma 2 exp 3 idle
   if (ROLE == 0) what = 0; else if (ROLE == 1) what = 1; else if (ROLE == 2) what = lo ? 0 : 1;
   else if (ROLE == 3) what = 2; else if (ROLE == 4) what = lo ? 1 : 2; else if (ROLE == 5) what = lo ? 0 : 3;
-  else if (ROLE == 6) what = lo ? 1 : 3; else what = lo ? 2 : 3;
+  else if (ROLE == 6) what = lo ? 1 : 3; else if (ROLE == 8) what = lo ? 0 : 2; else what = lo ? 2 : 3;
   f4 acc0 = {0,0,0,0}, acc1 = {0,0,0,0}, acc2={0,0,0,0}, acc3={0,0,0,0};
   float v[8];
   for (int i = 0; i < 8; ++i) v[i] = threadIdx.x * 0.001f + i;
@@ -74,5 +74,6 @@ int main() {
   printf("2 waves/SIMD EXP+EXP     %.3f ms\n", run<3>(iters, d));
   printf("2 waves/SIMD MFMA+FMA    %.3f ms\n", run<2>(iters, d));
   printf("2 waves/SIMD FMA+EXP     %.3f ms\n", run<4>(iters, d));
+  printf("2 waves/SIMD MFMA+EXP    %.3f ms\n", run<8>(iters, d));
   return 0;
 }
