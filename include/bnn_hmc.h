@@ -73,9 +73,10 @@ typedef struct bnnhmc_launch {
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */
   int threads;        /* threads per workgroup: 256, 512, 768 or 1024 (default 512 for MFMA,     */
                       /* 256 for FFMA)                                                           */
-  int pipeline;       /* MFMA tile loop: 0 or 2 = loads issued two tiles ahead with explicit     */
-                      /* waits (default), 1 = software-pipelined GEMM/pointwise stages,          */
-                      /* 3 = plain loop (default 1024 threads)                                   */
+  int pipeline;       /* MFMA tile loop: 0 = default; 2 = loads issued two tiles ahead with      */
+                      /* explicit waits (the default at 512 threads, built for 512 threads only),*/
+                      /* 1 = software-pipelined GEMM/pointwise stages (512 or 256 threads),      */
+                      /* 3 = plain loop (the default at other thread counts)                     */
   int transitions_per_launch; /* bound on one kernel's run time (default 8; 1 for 64 -> 128 -> 1) */
   unsigned spin_limit; /* polls before an in-kernel wait gives up (default 1 << 22)              */
 } bnnhmc_launch;

@@ -139,6 +139,9 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
   // MFMA tile loop: 0 / 2 = explicitly prefetched loop (default), 1 = software-pipelined, 3 = plain
   int loop = 0;
   if (l.layer == BNNHMC_LAYER_MFMA) loop = l.pipeline == 1 ? 1 : (l.pipeline == 3 ? 0 : 2);
+  // the prefetched loop exists for 512 threads only; other sizes get the plain loop unless the
+  // prefetched one was asked for by name (then there is no kernel, reported below)
+  if (l.layer == BNNHMC_LAYER_MFMA && l.pipeline == 0 && l.threads > 0 && l.threads != 512) loop = 0;
   p.wide = m.d0 == 64 && m.d1 == 128;
   if (p.wide) {
     if (l.layer != BNNHMC_LAYER_MFMA)

@@ -1128,8 +1128,11 @@ const void* hmc_kernel_for(int d0, int d1, int layer, int lik, int threads, int 
   using MA = MfmaLayer<22, 40, 2>;
   using F = FfmaLayer<22, 40>;
   if (layer == 0 && pipeline == 2) {
-    if (threads == 1024) return lik == 0 ? kernel_ptr<MA, 0, 1024>() : kernel_ptr<MA, 1, 1024>();
-    if (threads == 768) return lik == 0 ? kernel_ptr<MA, 0, 768>() : kernel_ptr<MA, 1, 768>();
+    // The prefetched loop is built for 512 threads only.  Its loads are issued from inline assembly
+    // and land in their registers long after the compiler believes them written: with fewer than
+    // 256 VGPRs per thread (768 or 1024 threads) the kernel spills, and a register that is spilled or
+    // re-used while its load is still in flight is corrupted.  The build checks that this kernel (and
+    // the wide-layer kernel, which loads the same way) has no spills.
     if (threads == 512) return lik == 0 ? kernel_ptr<MA, 0, 512>() : kernel_ptr<MA, 1, 512>();
   } else if (layer == 0 && pipeline == 1) {
     if (threads == 512) return lik == 0 ? kernel_ptr<MP, 0, 512>() : kernel_ptr<MP, 1, 512>();

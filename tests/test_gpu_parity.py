@@ -90,7 +90,7 @@ def test_eval_matches_oracle(pkg, lib, orc, layer, kind, n, G):
     s.close()
 
 
-@pytest.mark.parametrize("pipeline,threads", [(1, 512), (3, 512), (3, 1024), (2, 1024)])
+@pytest.mark.parametrize("pipeline,threads", [(1, 512), (3, 512), (3, 768), (3, 1024)])
 def test_alternative_tile_loops_match_oracle(pkg, lib, orc, pipeline, threads):
     """The software-pipelined (1) and plain (3) tile loops and other workgroup sizes stay selectable
     through the launch parameters; they must give the same gradients as the default loop."""
@@ -107,6 +107,15 @@ def test_alternative_tile_loops_match_oracle(pkg, lib, orc, pipeline, threads):
     ell_o, prior_o, grad_o, _ = orc.eval_f32(om, X, y, w)
     close_grad(grad, grad_o, "grad vs f32 oracle")
     np.testing.assert_allclose(ell, ell_o, rtol=RTOL, atol=RTOL * max(1.0, float(np.abs(ell_o).max())))
+
+
+def test_prefetched_loop_is_refused_where_it_would_spill(pkg, lib):
+    # the loop whose loads come from inline assembly is built for 512 threads only; asking for it by
+    # name with another workgroup size is an error, leaving the loop unspecified selects the plain one
+    with pytest.raises(pkg.BnnHmcError):
+        lib.create(lib.default_model(n=64), lib.default_hmc(), lib.default_launch(pipeline=2, threads=1024), 1, 1)
+    s = lib.create(lib.default_model(n=64), lib.default_hmc(), lib.default_launch(threads=1024), 1, 1)
+    s.close()
 
 
 def test_eval_is_deterministic_and_layout_agnostic(pkg, lib, orc):
