@@ -33,7 +33,10 @@ enum {
   BNNHMC_ERR_NO_DEVICE = 3, /* no gfx950 device visible                                           */
   BNNHMC_ERR_RESIDENCY = 4, /* the cooperating workgroups of one chain cannot all be resident     */
   BNNHMC_ERR_TIMEOUT = 5,   /* a bounded in-kernel wait expired; the launch was abandoned         */
-  BNNHMC_ERR_STATE = 6      /* call order violated (e.g. run before init_chains)                  */
+  BNNHMC_ERR_STATE = 6,     /* call order violated (e.g. run before init_chains)                  */
+  BNNHMC_ERR_DIVERGED = 7   /* the workgroups that share a chain did not all integrate the same   */
+                            /* state (each reports a hash of it after every launch); the results  */
+                            /* of the launch are not to be trusted                                */
 };
 
 enum { BNNHMC_LIK_STUDENT_T = 0, BNNHMC_LIK_GAUSSIAN = 1 };
@@ -71,12 +74,15 @@ typedef struct bnnhmc_launch {
                       /* device, up to 256 per chain), 256 for the step operator; the              */
                       /* 64 -> 128 -> 1 network takes at most 64                                    */
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */
-  int threads;        /* threads per workgroup: 256, 512, 768 or 1024 (default 512 for MFMA,     */
-                      /* 256 for FFMA)                                                           */
-  int pipeline;       /* MFMA tile loop: 0 = default; 2 = loads issued two tiles ahead with      */
-                      /* explicit waits (the default at 512 threads, built for 512 threads only),*/
+  int threads;        /* threads per workgroup; default 512 for MFMA (every tile loop), 256 for  */
+                      /* FFMA and with wgs_per_cu = 2.  The plain MFMA loop is also built for    */
+                      /* 256, 768 and 1024 threads (the last two leave too few registers and    */
+                      /* spill: correct, slower)                                                 */
+  int pipeline;       /* MFMA tile loop: 0 = default: loop 2 at 512 threads, loop 3 otherwise;   */
+                      /* 2 = loads issued two tiles ahead with explicit waits (512 threads only: */
+                      /* asking for it with another size is an error),                           */
                       /* 1 = software-pipelined GEMM/pointwise stages (512 or 256 threads),      */
-                      /* 3 = plain loop (the default at other thread counts)                     */
+                      /* 3 = plain loop (256, 512, 768 or 1024 threads)                          */
   int transitions_per_launch; /* bound on one kernel's run time (default 8; 1 for 64 -> 128 -> 1) */
   unsigned spin_limit; /* polls before an in-kernel wait gives up (default 1 << 22)              */
 } bnnhmc_launch;
@@ -114,8 +120,11 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
                      size_t workspace_bytes, float eps, int lp_steps, void* stream);
 
 /* Synchronises `stream` and reports whether the last bnnhmc_mcmc_step on this workspace ran to
- * completion (BNNHMC_ERR_TIMEOUT if a bounded in-kernel wait expired).  Stands in for the
- * CUDA_CHECK after the launch (include/mcmc/mcmc_step_ffma.h:412). */
+ * completion: BNNHMC_ERR_TIMEOUT if a bounded in-kernel wait expired (the outputs were then not
+ * written), BNNHMC_ERR_DIVERGED if the workgroups did not all hold the same state at the end.  Every
+ * bnnhmc_mcmc_step clears the record of the one before it, so check each step whose outcome matters.
+ * `launch` is not needed (the record sits at the start of the workspace) and may be NULL.  Stands in
+ * for the CUDA_CHECK after the launch (include/mcmc/mcmc_step_ffma.h:412). */
 int bnnhmc_step_check(const bnnhmc_model* model, const bnnhmc_launch* launch, void* workspace,
                       void* stream);
 
@@ -136,7 +145,7 @@ int bnnhmc_log_acpt(int n_loss, int n_mom, const float* prev_loss, const float* 
 
 /* Sums of the data log-likelihood (first n entries) and of the log-prior (next n_params entries) of
  * a loss_values vector.  Replaces get_loss_values (include/mcmc/kernel_helpers.h:190-216);
- * synchronises the stream. */
+ * synchronises the stream.  Allocates nothing; at most 64 calls may be in flight at once on a GPU. */
 int bnnhmc_get_loss_values(const float* loss_values, int n, int n_params, float* loss1_host,
                            float* loss2_host, void* stream);
 

@@ -15,7 +15,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG_DIR)
 LIB_PATH = os.path.join(PKG_DIR, "libbnn_hmc.so")
 
-OK, ERR_INVALID, ERR_HIP, ERR_NO_DEVICE, ERR_RESIDENCY, ERR_TIMEOUT, ERR_STATE = range(7)
+OK, ERR_INVALID, ERR_HIP, ERR_NO_DEVICE, ERR_RESIDENCY, ERR_TIMEOUT, ERR_STATE, ERR_DIVERGED = range(8)
 LIK_STUDENT_T, LIK_GAUSSIAN = 0, 1
 LAYER_MFMA, LAYER_FFMA = 0, 1
 STREAM_X, STREAM_TEACHER, STREAM_NOISE, STREAM_MOMENTUM, STREAM_ACCEPT = range(5)

@@ -33,6 +33,29 @@ hipError_t launch_fill_f32(float* p, size_t n, float v, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Runs after every launch of a trajectory kernel: all workgroups of a chain group must report the
+// same state hash.  The first mismatch is recorded in the status words ([4] workgroup index + 1,
+// [5] its chain group, [6..9] the two hashes); a launch that was abandoned (status[0] set) left no
+// hashes to compare.
+__global__ void compare_hashes_kernel(const unsigned long long* h, int wgs, int G, unsigned* status) {
+  if (status[0] != 0u) return;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < wgs; i += gridDim.x * blockDim.x) {
+    const int lead = i / G * G;
+    if (h[i] != h[lead] && atomicCAS(status + 4, 0u, (unsigned)i + 1u) == 0u) {
+      status[5] = (unsigned)(i / G);
+      status[6] = (unsigned)h[i];
+      status[7] = (unsigned)(h[i] >> 32);
+      status[8] = (unsigned)h[lead];
+      status[9] = (unsigned)(h[lead] >> 32);
+    }
+  }
+}
+hipError_t launch_compare_hashes(const unsigned long long* h, int wgs, int G, unsigned* status,
+                                 hipStream_t stream) {
+  hipLaunchKernelGGL(compare_hashes_kernel, dim3(1), dim3(256), 0, stream, h, wgs, G, status);
+  return hipGetLastError();
+}
+
 // main.h:207-216 with the counter-based generator
 __global__ void sample_momentum_kernel(uint32_t seed, uint32_t chain_id, uint32_t transition, int n,
                                        float* a, float* b) {

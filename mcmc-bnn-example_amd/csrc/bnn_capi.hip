@@ -7,8 +7,10 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "bnn_device.h"
@@ -45,6 +47,7 @@ int fail(int code, const char* fmt, ...) {
 ModelConsts make_consts(const bnnhmc_model& m) {
   const double pi = 3.14159265358979323846;
   ModelConsts c;
+  c.scale = (float)m.lik_scale;
   c.scale_recp = (float)(1.0 / m.lik_scale);
   c.df = (float)m.lik_df;
   c.df_recp = m.lik_kind == BNNHMC_LIK_STUDENT_T ? (float)(1.0 / m.lik_df) : 0.0f;
@@ -85,7 +88,7 @@ struct DeviceInfo {
   std::string arch;
 };
 
-int query_device(DeviceInfo& di) {
+int query_device_uncached(DeviceInfo& di) {
   int n = 0;
   hipError_t e = hipGetDeviceCount(&n);
   if (e != hipSuccess || n <= 0) {
@@ -101,6 +104,22 @@ int query_device(DeviceInfo& di) {
   if (di.arch.rfind("gfx950", 0) != 0)
     return fail(BNNHMC_ERR_NO_DEVICE, "device 0 is %s; this library is built for gfx950 only",
                 di.arch.c_str());
+  return BNNHMC_OK;
+}
+
+// The device is queried once per process; failures are not cached (a later call asks again).
+std::mutex g_cache_mutex;
+bool g_device_known = false;
+DeviceInfo g_device;
+
+int query_device(DeviceInfo& di) {
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  if (!g_device_known) {
+    const int rc = query_device_uncached(g_device);
+    if (rc) return rc;
+    g_device_known = true;
+  }
+  di = g_device;
   return BNNHMC_OK;
 }
 
@@ -120,7 +139,7 @@ struct Plan {
   int transitions_per_launch = 8;
 };
 
-int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& di, Plan& p) {
+int make_plan_uncached(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& di, Plan& p) {
   bnnhmc_launch l;
   bnnhmc_default_launch(&l);
   if (lp) {
@@ -153,7 +172,7 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
     p.kernel = hmc_kernel_wide_for(m.d0, m.d1, m.lik_kind, p.threads, &p.dyn_lds, &p.wg_scratch_floats);
   } else {
     p.threads = l.threads > 0 ? l.threads
-                              : (l.layer == BNNHMC_LAYER_FFMA || l.wgs_per_cu == 2 ? 256 : (loop == 0 ? 1024 : 512));
+                              : (l.layer == BNNHMC_LAYER_FFMA || l.wgs_per_cu == 2 ? 256 : 512);
     p.kernel = hmc_kernel_for(m.d0, m.d1, l.layer, m.lik_kind, p.threads, loop);
   }
   if (!p.kernel)
@@ -183,35 +202,97 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
   return BNNHMC_OK;
 }
 
+// Plans are kept per (layer sizes, likelihood, launch parameters): the occupancy query and the
+// function-attribute call are made once, so that the step operator touches no device property on
+// later calls (the reference's operator does nothing but launch, mcmc_step_ffma.h:395-427).
+struct PlanKey {
+  int d0, d1, lik, layer, cus_per_chain, wgs_per_cu, threads, pipeline, tpl;
+  unsigned spin_limit;
+  bool operator==(const PlanKey& o) const {
+    return d0 == o.d0 && d1 == o.d1 && lik == o.lik && layer == o.layer &&
+           cus_per_chain == o.cus_per_chain && wgs_per_cu == o.wgs_per_cu && threads == o.threads &&
+           pipeline == o.pipeline && tpl == o.tpl && spin_limit == o.spin_limit;
+  }
+};
+std::vector<std::pair<PlanKey, Plan>> g_plans;
+
+int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& di, Plan& p) {
+  bnnhmc_launch l;
+  memset(&l, 0, sizeof(l));
+  if (lp) l = *lp;
+  const PlanKey key{m.d0, m.d1, m.lik_kind, l.layer, l.cus_per_chain, l.wgs_per_cu, l.threads,
+                    l.pipeline, l.transitions_per_launch, l.spin_limit};
+  {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    for (const auto& e : g_plans)
+      if (e.first == key) {
+        p = e.second;
+        return BNNHMC_OK;
+      }
+  }
+  const int rc = make_plan_uncached(m, lp, di, p);
+  if (rc) return rc;
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  g_plans.emplace_back(key, p);
+  return BNNHMC_OK;
+}
+
 // Exchange scratch: partial records for `wgs` co-resident workgroups (double-buffered), one totals
 // record and one barrier line per chain group (at most `groups`), status words.
 size_t workspace_bytes_for(int P, int wgs, int groups) {
   const size_t slot = (size_t)partial_slot_floats(P);
-  size_t bytes = (size_t)wgs * 2 * slot * sizeof(float);
+  size_t bytes = STATUS_WORDS * sizeof(unsigned);
+  bytes += (size_t)(wgs + 31) / 32 * 32 * sizeof(unsigned long long);
+  bytes += (size_t)wgs * 2 * slot * sizeof(float);
   bytes += (size_t)groups * slot * sizeof(float);
   bytes += (size_t)groups * BARRIER_STRIDE_WORDS * sizeof(unsigned);
-  bytes += 64 * sizeof(unsigned);
   return bytes;
 }
 
+// The status words come first and the state hashes right behind them, so that both are found
+// without knowing how the rest of the scratch is divided.
 struct Workspace {
+  unsigned* status;
+  unsigned long long* rank_hash;
   float* partials;
   float* totals;
   unsigned* barrier;
-  unsigned* status;
 };
 Workspace carve_workspace(void* base, int P, int wgs, int groups) {
   Workspace w;
   char* b = (char*)base;
   const size_t slot = (size_t)partial_slot_floats(P);
+  w.status = (unsigned*)b;
+  b += STATUS_WORDS * sizeof(unsigned);
+  w.rank_hash = (unsigned long long*)b;
+  b += (size_t)(wgs + 31) / 32 * 32 * sizeof(unsigned long long);
   w.partials = (float*)b;
   b += (size_t)wgs * 2 * slot * sizeof(float);
   w.totals = (float*)b;
   b += (size_t)groups * slot * sizeof(float);
   w.barrier = (unsigned*)b;
-  b += (size_t)groups * BARRIER_STRIDE_WORDS * sizeof(unsigned);
-  w.status = (unsigned*)b;
   return w;
+}
+
+// Synchronises `stream` and reads the status words the launches on it have left since the words
+// were last cleared: BNNHMC_ERR_TIMEOUT if a bounded wait expired, BNNHMC_ERR_DIVERGED if the
+// workgroups of a chain group did not all hold the same state at the end of a launch.
+int read_status(void* workspace, hipStream_t stream) {
+  unsigned st[16] = {0};
+  HIP_TRY(hipMemcpyAsync(st, workspace, sizeof(st), hipMemcpyDeviceToHost, stream));
+  HIP_TRY(hipStreamSynchronize(stream));
+  if (st[0] != 0)
+    return fail(BNNHMC_ERR_TIMEOUT,
+                "a workgroup (%u) waited longer than the spin limit for its chain group; the launch "
+                "was abandoned",
+                st[1] ? st[1] - 1 : 0u);
+  if (st[4] != 0)
+    return fail(BNNHMC_ERR_DIVERGED,
+                "workgroup %u (chain group %u of its launch) integrated a different state than the first "
+                "workgroup of its group (state hash %08x%08x vs %08x%08x): a partial record was read before "
+                "it was complete",
+                st[4] - 1, st[5], st[7], st[6], st[9], st[8]);
+  return BNNHMC_OK;
 }
 
 // Workgroups per chain for a batch of `groups` chains: the configured count, widened by powers of
@@ -240,6 +321,14 @@ int debug_drop_rank() {
   return e && *e ? atoi(e) : -1;
 }
 
+// Test hook: BNNHMC_DEBUG_PERTURB_HASH=<rank> makes that rank of every chain group flip one bit of
+// the state hash it reports (its memory traffic and its results are untouched), so that the
+// comparison of the hashes fails.  Unset in normal use.
+int debug_perturb_hash_rank() {
+  const char* e = getenv("BNNHMC_DEBUG_PERTURB_HASH");
+  return e && *e ? atoi(e) : -1;
+}
+
 // host restatement of the hidden activation (kernel_helpers.h:34-42) for the data generator
 inline float host_tanh(float x) {
   const float e = exp2f(x * -2.88539008177792681472f);
@@ -247,14 +336,11 @@ inline float host_tanh(float x) {
   return std::fabs(x) < 0.0048176045529544353485f ? x : fmaf(sigm, 2.0f, -1.0f);
 }
 
-void generate_window_host(uint32_t seed, uint32_t window, int n, int d0, int d1, float teacher_scale,
-                          float noise_sigma, float* X, float* y, float* teacher) {
+void generate_rows(uint32_t seed, uint32_t window, int row_begin, int row_end, int d0, int d1,
+                   float noise_sigma, const std::vector<float>& th, float* X, float* y) {
   const Layout L = make_layout(d0, d1);
-  std::vector<float> th(L.P), h(d1);
-  for (int p = 0; p < L.P; ++p)
-    th[p] = teacher_scale * rng_normal(seed, window, STREAM_TEACHER, 0, (uint64_t)p);
-  if (teacher) memcpy(teacher, th.data(), sizeof(float) * L.P);
-  for (int i = 0; i < n; ++i) {
+  std::vector<float> h(d1);
+  for (int i = row_begin; i < row_end; ++i) {
     float* x = X + (size_t)i * d0;
     for (int k = 0; k < d0; ++k) x[k] = rng_normal(seed, window, STREAM_X, 0, (uint64_t)i * d0 + k);
     for (int c = 0; c < d1; ++c) h[c] = th[L.ob1 + c];
@@ -266,6 +352,56 @@ void generate_window_host(uint32_t seed, uint32_t window, int n, int d0, int d1,
   }
 }
 
+// Every element is a function of (seed, window, its index) alone, so the rows can be filled by any
+// number of threads with the same result.
+void generate_window_host(uint32_t seed, uint32_t window, int n, int d0, int d1, float teacher_scale,
+                          float noise_sigma, float* X, float* y, float* teacher) {
+  const Layout L = make_layout(d0, d1);
+  std::vector<float> th(L.P);
+  for (int p = 0; p < L.P; ++p)
+    th[p] = teacher_scale * rng_normal(seed, window, STREAM_TEACHER, 0, (uint64_t)p);
+  if (teacher) memcpy(teacher, th.data(), sizeof(float) * L.P);
+  unsigned hw = std::thread::hardware_concurrency();
+  const int n_threads = (int)std::max(1u, std::min({hw ? hw : 1u, 16u, (unsigned)(n / 4096 + 1)}));
+  if (n_threads == 1) {
+    generate_rows(seed, window, 0, n, d0, d1, noise_sigma, th, X, y);
+    return;
+  }
+  std::vector<std::thread> pool;
+  for (int t = 0; t < n_threads; ++t) {
+    const int b = (int)((long)n * t / n_threads), e = (int)((long)n * (t + 1) / n_threads);
+    pool.emplace_back(generate_rows, seed, window, b, e, d0, d1, noise_sigma, std::cref(th), X, y);
+  }
+  for (auto& t : pool) t.join();
+}
+
+}  // namespace
+
+// Result slots of bnnhmc_get_loss_values: a static device array (every GPU holds its own copy), whose
+// address on the current device is looked up once per device.
+constexpr int LOSS_SLOTS = 64;
+constexpr int MAX_DEVICES = 16;
+static __device__ __align__(256) float g_loss_slots[LOSS_SLOTS][2];
+
+namespace {
+float* g_loss_slots_ptr[MAX_DEVICES] = {nullptr};
+unsigned g_loss_next = 0;
+
+int loss_slot(float** out) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= MAX_DEVICES)
+    return fail(BNNHMC_ERR_INVALID, "device index %d is beyond the %d this library keeps state for", dev,
+                MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  if (!g_loss_slots_ptr[dev]) {
+    void* p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_loss_slots)));
+    g_loss_slots_ptr[dev] = (float*)p;
+  }
+  *out = g_loss_slots_ptr[dev] + 2 * (size_t)(g_loss_next++ % LOSS_SLOTS);
+  return BNNHMC_OK;
+}
 }  // namespace
 
 // =================================================================================================
@@ -345,11 +481,13 @@ KArgs base_args(const bnnhmc_sampler* s) {
   a.L = s->hmc.leapfrog_steps;
   a.spin_limit = s->plan.spin_limit;
   a.debug_drop_rank = debug_drop_rank();
+  a.debug_perturb_hash_rank = debug_perturb_hash_rank();
   Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups);
   a.partials = w.partials;
   a.totals = w.totals;
   a.barrier = w.barrier;
   a.status = w.status;
+  a.rank_hash = w.rank_hash;
   a.wg_scratch = s->wg_scratch;
   return a;
 }
@@ -360,24 +498,21 @@ int launch_and_count(bnnhmc_sampler* s, KArgs& a, int groups) {
            &wgs);
   HIP_TRY(launch_fill_u32(a.barrier, (size_t)groups * BARRIER_STRIDE_WORDS, 0u, s->stream));
   HIP_TRY(launch_hmc_kernel(s->plan.kernel, a, wgs, s->plan.threads, s->plan.dyn_lds, s->stream));
+  HIP_TRY(launch_compare_hashes(a.rank_hash, wgs, a.G, a.status, s->stream));
   s->last_workgroups = wgs;
   return BNNHMC_OK;
 }
 
 int check_status(bnnhmc_sampler* s) {
-  Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups);
-  unsigned st[2] = {0, 0};
-  HIP_TRY(hipMemcpyAsync(st, w.status, sizeof(st), hipMemcpyDeviceToHost, s->stream));
-  HIP_TRY(hipStreamSynchronize(s->stream));
-  if (st[0] != 0) {
-    HIP_TRY(launch_fill_u32(w.status, 2, 0u, s->stream));
+  const int rc = read_status(s->workspace, s->stream);
+  if (rc == BNNHMC_ERR_TIMEOUT || rc == BNNHMC_ERR_DIVERGED) {
+    // the words are sticky until cleared: the sampler stays usable after the error is reported
+    const std::string msg = g_last_error;
+    HIP_TRY(launch_fill_u32((unsigned*)s->workspace, STATUS_WORDS, 0u, s->stream));
     HIP_TRY(hipStreamSynchronize(s->stream));
-    return fail(BNNHMC_ERR_TIMEOUT,
-                "a workgroup (%u) waited longer than the spin limit for its chain group; the launch "
-                "was abandoned",
-                st[1] ? st[1] - 1 : 0u);
+    g_last_error = msg;
   }
-  return BNNHMC_OK;
+  return rc;
 }
 
 // evaluate MODE_STEPS with L = 1, eps = 0 for `groups` parameter vectors starting at w_dev
@@ -593,37 +728,29 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
   a.prior_out = loss_values + model->n;
   a.spin_limit = plan.spin_limit;
   a.debug_drop_rank = debug_drop_rank();
+  a.debug_perturb_hash_rank = debug_perturb_hash_rank();
   Workspace w = carve_workspace(workspace, L.P, G, 1);
   a.partials = w.partials;
   a.totals = w.totals;
   a.barrier = w.barrier;
   a.status = w.status;
+  a.rank_hash = w.rank_hash;
   int wgs = 0;
   set_grid(a, 1, G, &wgs);
-  // barrier and status words start from zero on every call
-  HIP_TRY(launch_fill_u32(w.barrier, BARRIER_STRIDE_WORDS + 64, 0u, st));
+  // status and barrier words start from zero on every call
+  HIP_TRY(launch_fill_u32(w.status, STATUS_WORDS, 0u, st));
+  HIP_TRY(launch_fill_u32(w.barrier, BARRIER_STRIDE_WORDS, 0u, st));
   HIP_TRY(launch_hmc_kernel(plan.kernel, a, wgs, plan.threads, plan.dyn_lds, st));
+  HIP_TRY(launch_compare_hashes(a.rank_hash, wgs, G, a.status, st));
   return BNNHMC_OK;
 }
 
 int bnnhmc_step_check(const bnnhmc_model* model, const bnnhmc_launch* launch, void* workspace,
                       void* stream) {
+  (void)launch;
   if (!model || !workspace) return fail(BNNHMC_ERR_INVALID, "null argument to bnnhmc_step_check");
-  int G = launch && launch->cus_per_chain > 0 ? launch->cus_per_chain : 0;
-  if (G == 0) {
-    DeviceInfo di;
-    int rc = query_device(di);
-    if (rc) return rc;
-    G = step_group(launch, di.cus, model->d0 == 64 ? 64 : 256);
-  }
-  Workspace w = carve_workspace(workspace, make_layout(model->d0, model->d1).P, G, 1);
-  unsigned st[2] = {0, 0};
-  HIP_TRY(hipMemcpyAsync(st, w.status, sizeof(st), hipMemcpyDeviceToHost, (hipStream_t)stream));
-  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-  if (st[0] != 0)
-    return fail(BNNHMC_ERR_TIMEOUT, "workgroup %u waited longer than the spin limit; step abandoned",
-                st[1] ? st[1] - 1 : 0u);
-  return BNNHMC_OK;
+  // the status words sit at the start of the workspace whatever the launch parameters were
+  return read_status(workspace, (hipStream_t)stream);
 }
 
 int bnnhmc_sample_momentum(uint32_t seed, uint32_t chain_id, uint32_t transition, int n,
@@ -657,14 +784,16 @@ int bnnhmc_get_loss_values(const float* loss_values, int n, int n_params, float*
   if (!loss_values || n < 0 || n_params < 0)
     return fail(BNNHMC_ERR_INVALID, "bad arguments to bnnhmc_get_loss_values");
   hipStream_t st = (hipStream_t)stream;
+  // No allocation (the reference allocates its reduction scratch once, kernel_helpers.h:194-204):
+  // the two sums land in one of LOSS_SLOTS pairs of a static device array, handed out round-robin; a
+  // pair is in use only until this call returns, so up to LOSS_SLOTS calls may overlap.
   float* d = nullptr;
-  HIP_TRY(hipMalloc((void**)&d, 2 * sizeof(float)));
-  hipError_t e = launch_loss_sums(loss_values, n, n_params, d, st);
+  int rc = loss_slot(&d);
+  if (rc) return rc;
+  HIP_TRY(launch_loss_sums(loss_values, n, n_params, d, st));
   float h[2] = {0, 0};
-  if (e == hipSuccess) e = hipMemcpyAsync(h, d, sizeof(h), hipMemcpyDeviceToHost, st);
-  if (e == hipSuccess) e = hipStreamSynchronize(st);
-  (void)hipFree(d);
-  if (e != hipSuccess) return fail(BNNHMC_ERR_HIP, "loss sums failed: %s", hipGetErrorString(e));
+  HIP_TRY(hipMemcpyAsync(h, d, sizeof(h), hipMemcpyDeviceToHost, st));
+  HIP_TRY(hipStreamSynchronize(st));
   if (loss1_host) *loss1_host = h[0];
   if (loss2_host) *loss2_host = h[1];
   return BNNHMC_OK;

@@ -24,6 +24,7 @@ inline Layout make_layout(int d0, int d1) {
 // float constants of the likelihood and the prior, derived on the host exactly as the reference
 // derives them from its double constexprs (mcmc_step_ffma.h:289-300, 113-118)
 struct ModelConsts {
+  float scale;       // lik_scale
   float scale_recp;  // 1 / lik_scale
   float df;
   float df_recp;
@@ -44,6 +45,19 @@ enum KernelMode : int {
 // multiple of 4, then 4 words of which the first two hold a double (sum of per-row log-likelihood
 // terms); rounded up to whole 128-byte lines so that a 32-parameter slice of a record is one line.
 inline int partial_slot_floats(int P) { return (((P + 3) / 4) * 4 + 4 + 31) / 32 * 32; }
+
+// status words at the start of the exchange scratch (64 are reserved)
+constexpr int STATUS_WORDS = 64;
+
+// 64-bit mixing function of the state hash (the finaliser of splitmix64)
+#if defined(__HIPCC__)
+__host__ __device__
+#endif
+inline unsigned long long mix64(unsigned long long z) {
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
 
 // barrier words per chain group: the group's counter, eight block counters (one per 32 ranks, used by
 // groups of more than 64 workgroups) and the counters of the second barrier of the two-phase
@@ -114,10 +128,13 @@ struct KArgs {
   float* totals;       // [group][slot]: reduced gradient, two-phase reduction only
   int two_phase;       // 1: each workgroup reduces a slice of the parameters, then all read the totals
   unsigned* barrier;   // [group][BARRIER_STRIDE_WORDS]
-  unsigned* status;    // [0] abort flag, [1] timed-out workgroup + 1
+  unsigned* status;    // [0] abort flag, [1] timed-out workgroup + 1; [4..9] belong to the hash check
+  unsigned long long* rank_hash;  // [workgroup in group-major order]: hash of the state this workgroup
+                                  // integrated; all workgroups of a chain group must agree
   unsigned spin_limit;
   float* wg_scratch;   // wide-layer kernel, MODE_TRANSITIONS: [workgroup][3][P_AL] accepted w, g and start momentum
   int debug_drop_rank; // >= 0: this rank of every group never signals arrival (exercises the timeout path)
+  int debug_perturb_hash_rank;  // >= 0: this rank of every group flips a bit of its state hash
   unsigned* debug_xcc; // optional [workgroup] XCC id
   unsigned long long* debug_phase;  // optional [workgroup][10]: cycles per phase of a step, launch ticks
 };

@@ -67,12 +67,19 @@ struct MfmaLayer {
   static constexpr int oB1 = D0 * D1, oW2 = oB1 + D1, oB2 = oW2 + D1, P = oB2 + 1;
   static constexpr int P_AL = (P + 3) / 4 * 4;
 
-  float w1b[KS][NT];   // W1_aug scaled by -2/ln 2: GEMM1 yields the exp2 argument of the activation
-  float w2v[NT];       // w2[c]
-  float w2y[NT];       // -w2[c] / lik_scale: the layer-2 dot yields the scaled residual directly
-  float yh_init;       // -b2 / lik_scale in lane n == 0, else 0
-  f4 dacc[NT][2];
-  float dw2acc[NT];
+  // The activation is carried as the logistic value s = 1 / (1 + 2^t) = (h + 1) / 2 and h = tanh is
+  // never formed: the layer-2 dot, the layer-2 weight gradient and 1 - h^2 = 4 s (1 - s) are all
+  // affine in s or products of s, and the constants move into per-step operands (one VALU
+  // instruction less per hidden value and row).
+  float w1b[KS][NT];   // W1_aug scaled by -2/ln 2: GEMM1 yields the exp2 argument t of the activation
+  float w2g[NT];       // -2 w2[c] k with k = 1/scale^2 (Gaussian: the layer-2 dot yields the per-row
+                       // loss gradient g directly) or 1/scale (Student-t: it yields the scaled residual)
+  float y_k;           // k in lane n == 0, else 0
+  float y_0;           // (sum_c w2[c] - b2) k in lane n == 0, else 0: the constant part of the dot
+  f4 dacc[NT][2];      // sum over rows of s (1 - s) g x_aug: dW1_aug^T / (4 w2[c])
+  float dw2s[NT];      // sum over rows of g s
+  float gacc;          // sum over rows of g, added in the order of dw2s: dw2 = 2 dw2s - gacc is then
+                       // exactly zero where every s is 1/2 (all weights zero, the reference's start)
   double dl;
 
   struct TileIn {
@@ -83,8 +90,11 @@ struct MfmaLayer {
 
   static constexpr float kExp2Scale = -2.88539008177792681472f;  // -2 / ln 2, kernel_helpers.h:37
 
+  template <int LIK>
   __device__ __forceinline__ void load_weights(const float* s_w, const ModelConsts& mc) {
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    const float k = LIK == 1 ? mc.scale_recp * mc.scale_recp : mc.scale_recp;
+    float w2sum = 0.0f;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int c = 16 * t + n;
@@ -92,16 +102,19 @@ struct MfmaLayer {
       const int cc = cv ? c : 0;
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
-        const int k = KS * q + s;
+        const int kk = KS * q + s;
         float v = 0.0f;
-        if (k < D0) v = s_w[k * D1 + cc];
-        else if (k == D0) v = s_w[oB1 + cc];
+        if (kk < D0) v = s_w[kk * D1 + cc];
+        else if (kk == D0) v = s_w[oB1 + cc];
         w1b[s][t] = cv ? v * kExp2Scale : 0.0f;
       }
-      w2v[t] = cv ? s_w[oW2 + cc] : 0.0f;
-      w2y[t] = -w2v[t] * mc.scale_recp;
+      const float w2c = cv ? s_w[oW2 + cc] : 0.0f;
+      w2sum += w2c;
+      w2g[t] = -2.0f * w2c * k;
     }
-    yh_init = n == 0 ? -s_w[oB2] * mc.scale_recp : 0.0f;
+    w2sum = row16_allreduce(w2sum);  // sum over all hidden units, the same bits in every lane
+    y_k = n == 0 ? k : 0.0f;
+    y_0 = n == 0 ? (w2sum - s_w[oB2]) * k : 0.0f;
   }
 
   __device__ __forceinline__ void zero_acc() {
@@ -109,8 +122,9 @@ struct MfmaLayer {
     for (int t = 0; t < NT; ++t) {
       dacc[t][0] = f4{0.f, 0.f, 0.f, 0.f};
       dacc[t][1] = f4{0.f, 0.f, 0.f, 0.f};
-      dw2acc[t] = 0.0f;
+      dw2s[t] = 0.0f;
     }
+    gacc = 0.0f;
     dl = 0.0;
   }
 
@@ -157,40 +171,50 @@ struct MfmaLayer {
     }
   }
 
-  // C: activation, layer-2 dot, per-row loss gradient, layer-2 weight gradient, delta (in place).
-  // acc arrives as the exp2 argument t = -2 x / ln 2 of tanh(x) = 2 / (1 + 2^t) - 1
+  // C: activation, layer-2 dot, per-row loss gradient, layer-2 weight gradient, the two GEMM2
+  // operands.  acc arrives as the exp2 argument t = -2 x / ln 2 of s = 1 / (1 + 2^t), tanh(x) = 2 s - 1
   // (kernel_helpers.h:34-42 without its small-|x| identity branch, which changes the value by less
-  // than 1.5e-7).  delta leaves without the factor w2[c], which is applied once per step to the
-  // GEMM2 result; the padded hidden units (zero weights: h = 0) then carry delta = g, so the
-  // constant-one column of GEMM2 delivers db2 in row c = D1 for free.
+  // than 1.5e-7), and leaves as s (1 - s) = (1 - tanh^2) / 4.  The factors g (per row) and 4 w2[c]
+  // (per hidden unit) of delta = (1 - h^2) w2[c] g (kernel_helpers.h:43, mcmc_step_ffma.h:323) are
+  // applied to the other GEMM2 operand (xg = g x_aug: 8 products per tile instead of 12) and once
+  // per step to the GEMM2 result.  The padded hidden units (zero weights: s = 1/2) carry 1/4, so the
+  // constant-one column of GEMM2 delivers sum(g) / 4 = db2 / 4 in row c = D1 for free.
   template <int LIK, bool LAST, bool FULL>
-  __device__ __forceinline__ void pointwise(f4 (&acc)[NT], const f4& yv, const StepCtx& cx,
-                                            const ModelConsts& mc, int row0, int n, int q) {
-    float yh[4] = {yh_init, yh_init, yh_init, yh_init};
+  __device__ __forceinline__ void pointwise(f4 (&acc)[NT], const f4& yv, const f2 (&xb)[4],
+                                            f2 (&xg)[4], const StepCtx& cx, const ModelConsts& mc,
+                                            int row0, int n, int q) {
+    float yh[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) yh[j] = __builtin_fmaf(yv[j], y_k, y_0);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float e = __builtin_amdgcn_exp2f(acc[t][j]);
         const float sg = __builtin_amdgcn_rcpf(1.0f + e);
-        const float h = __builtin_fmaf(sg, 2.0f, -1.0f);
-        acc[t][j] = h;
-        yh[j] = __builtin_fmaf(w2y[t], h, yh[j]);
+        acc[t][j] = sg;
+        yh[j] = __builtin_fmaf(w2g[t], sg, yh[j]);
       }
     }
     float g[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      // scaled residual (y - yhat - b2) / scale, mcmc_step_ffma.h:293
-      const float diff = __builtin_fmaf(yv[j], mc.scale_recp, row16_allreduce(yh[j]));
-      float gj;
-      if (LIK == 0) gj = diff * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(diff, diff, mc.df));
-      else gj = diff * mc.scale_recp;
+      // (y - yhat - b2) k: the loss gradient (Gaussian) or the scaled residual (Student-t),
+      // mcmc_step_ffma.h:293-301
+      const float r = row16_allreduce(yh[j]);
+      float gj, diff;
+      if (LIK == 0) {
+        diff = r;
+        gj = diff * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(diff, diff, mc.df));
+      } else {
+        gj = r;
+      }
       const bool valid = FULL || (row0 + 4 * q + j < cx.n);
       gj = valid ? gj : 0.0f;  // mcmc_step_ffma.h:301
       g[j] = gj;
       if (LAST) {
         if (n == 0 && valid) {
+          if (LIK == 1) diff = r * mc.scale;
           const int row = row0 + 4 * q + j;
           const float lv = lik_value<LIK>(mc, diff);
           const float prev = cx.ell_prev ? cx.ell_prev[row] : 0.0f;
@@ -200,17 +224,21 @@ struct MfmaLayer {
       }
     }
 #pragma unroll
+    for (int j = 0; j < 4; ++j) gacc += g[j];
+#pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float h = acc[t][j];
-        dw2acc[t] = __builtin_fmaf(g[j], h, dw2acc[t]);
-        acc[t][j] = __builtin_fmaf(-h, h, 1.0f) * g[j];
+        const float sg = acc[t][j];
+        dw2s[t] = __builtin_fmaf(g[j], sg, dw2s[t]);
+        acc[t][j] = __builtin_fmaf(-sg, sg, sg);
       }
     }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xg[j] = xb[j] * g[j];
   }
 
-  // D: GEMM2, dW1_aug^T += delta^T X_aug
+  // D: GEMM2, dacc += (s (1 - s))^T (g X_aug)
   __device__ __forceinline__ void gemm2(const f4 (&dlt)[NT], const f2 (&xb)[4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -272,14 +300,15 @@ struct MfmaLayer {
       load(t2, i + 2 < te ? i + 2 : te - 1);
       gemm1(t1.xa, acc_nxt);                                       // tile i + 1
       gemm2(dlt_prev, xb_prev);                                    // tile i - 1 (zero delta at i = tb)
-      pointwise<LIK, LAST, true>(acc_cur, t0.yv, cx, mc, i * 16, n, q);  // tile i -> delta in acc_cur
+      f2 xg[4];
+      pointwise<LIK, LAST, true>(acc_cur, t0.yv, t0.xb, xg, cx, mc, i * 16, n, q);  // tile i
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         dlt_prev[t] = acc_cur[t];
         acc_cur[t] = acc_nxt[t];
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xb_prev[j] = t0.xb[j];
+      for (int j = 0; j < 4; ++j) xb_prev[j] = xg[j];
       t0 = t1;
       t1 = t2;
     }
@@ -320,9 +349,10 @@ struct MfmaLayer {
     for (int i = tb; i < te; ++i) {
       load(nx2, i + 2 < te ? i + 2 : te - 1);
       f4 acc[NT];
+      f2 xg[4];
       gemm1(cur.xa, acc);
-      pointwise<LIK, LAST, true>(acc, cur.yv, cx, mc, i * 16, n, q);
-      gemm2(acc, cur.xb);
+      pointwise<LIK, LAST, true>(acc, cur.yv, cur.xb, xg, cx, mc, i * 16, n, q);
+      gemm2(acc, xg);
       cur = nx1;
       nx1 = nx2;
     }
@@ -370,7 +400,7 @@ struct MfmaLayer {
     const f2 const_a = f2{1.0f, 0.0f};
     const f2 const_b = f2{2 * n == D0 ? 1.0f : 0.0f, 0.0f};
     int nxt = tb;  // tiles are issued in order, one call each; past the last tile the base stays
-    auto issue = [&](TileRaw& t, int) {  // exactly 7 loads
+    auto issue = [&](TileRaw& t) {  // exactly 7 loads
       const int tile = nxt < te ? nxt : te - 1;
       ++nxt;
       const float* bx = cx.X + (size_t)tile * (16 * D0);
@@ -378,26 +408,29 @@ struct MfmaLayer {
       // One block for the seven loads.  The leading s_nop gives the five wait states a memory
       // instruction needs after a VALU instruction wrote one of its SGPR operands (the compiler
       // reloads spilled SGPRs with v_readlane and does not see the loads inside the assembly, so it
-      // would not insert them itself).  The pure outputs are early-clobber: a returning load must
-      // not land in a register that still holds an offset of a load not yet issued.
+      // would not insert them itself).  EXEC is saved on entry and put back.  The pure outputs are
+      // early-clobber: a returning load must not land in a register that still holds an offset of a
+      // load not yet issued.
+      unsigned long long exec_save;
       asm volatile(
-          "s_nop 4\n\t"
+          "s_mov_b64 %[sv], exec\n\t"
+          "s_nop 3\n\t"
           "global_load_dwordx4 %[xa01], %[oa], %[bx]\n\t"
-          "s_mov_b64 exec, %[ma]\n\t"
+          "s_and_b64 exec, %[sv], %[ma]\n\t"
           "global_load_dwordx2 %[xa2], %[ol], %[bx]\n\t"
-          "s_mov_b64 exec, %[mb]\n\t"
+          "s_and_b64 exec, %[sv], %[mb]\n\t"
           "global_load_dwordx2 %[xb0], %[ob], %[bx]\n\t"
           "global_load_dwordx2 %[xb1], %[ob], %[bx] offset:%[r1]\n\t"
           "global_load_dwordx2 %[xb2], %[ob], %[bx] offset:%[r2]\n\t"
           "global_load_dwordx2 %[xb3], %[ob], %[bx] offset:%[r3]\n\t"
-          "s_mov_b64 exec, -1\n\t"
+          "s_mov_b64 exec, %[sv]\n\t"
           "global_load_dwordx4 %[yv], %[oy], %[by]"
           : [xa01] "=&v"(t.xa01), [xa2] "+v"(t.xa2), [xb0] "+v"(t.xb[0]), [xb1] "+v"(t.xb[1]),
-            [xb2] "+v"(t.xb[2]), [xb3] "+v"(t.xb[3]), [yv] "=&v"(t.yv)
+            [xb2] "+v"(t.xb[2]), [xb3] "+v"(t.xb[3]), [yv] "=&v"(t.yv), [sv] "=&s"(exec_save)
           : [oa] "v"(oa), [ol] "v"(ol), [ob] "v"(ob), [oy] "v"(oy), [bx] "s"(bx), [by] "s"(by),
             [ma] "s"(mask_a), [mb] "s"(mask_b), [r1] "n"(D0 * 4), [r2] "n"(2 * D0 * 4),
             [r3] "n"(3 * D0 * 4)
-          : "memory");
+          : "memory", "scc");
     };
     auto preset = [&](TileRaw& t) {
       t.xa2 = const_a;
@@ -405,35 +438,39 @@ struct MfmaLayer {
       for (int j = 0; j < 4; ++j) t.xb[j] = const_b;
     };
     auto compute = [&](TileRaw& t, int tile) {
-      wait_tile<14>(t);
       const f2 xa[KP] = {f2{t.xa01[0], t.xa01[1]}, f2{t.xa01[2], t.xa01[3]}, t.xa2};
       f4 acc[NT];
+      f2 xg[4];
       gemm1(xa, acc);
-      pointwise<LIK, LAST, true>(acc, t.yv, cx, mc, tile * 16, n, q);
-      gemm2(acc, t.xb);
+      pointwise<LIK, LAST, true>(acc, t.yv, t.xb, xg, cx, mc, tile * 16, n, q);
+      gemm2(acc, xg);
     };
     TileRaw A, B, C;
     preset(A);
     preset(B);
     preset(C);
-    issue(A, tb);
-    issue(B, tb + 1);
-    for (int i = tb; i < te; i += 3) {
-      issue(C, i + 2);
+    issue(A);
+    issue(B);
+    // steady state: three tiles per trip, every issue and every wait unconditional
+    int i = tb;
+    for (; i + 3 <= te; i += 3) {
+      issue(C);
+      wait_tile<14>(A);
       compute(A, i);
-      if (i + 1 < te) {
-        issue(A, i + 3);
-        compute(B, i + 1);
-      }
-      if (i + 2 < te) {
-        issue(B, i + 4);
-        compute(C, i + 2);
-      }
+      issue(A);
+      wait_tile<14>(B);
+      compute(B, i + 1);
+      issue(B);
+      wait_tile<14>(C);
+      compute(C, i + 2);
     }
-    // no register of a set may be reused before its last load has landed
+    // no register of a set may be used or reused before its last load has landed
     wait_tile<0>(A);
     wait_tile<0>(B);
     wait_tile<0>(C);
+    // the one or two tiles left over: A and B hold them (issued at the end of the last trip)
+    if (i < te) compute(A, i);
+    if (i + 1 < te) compute(B, i + 1);
   }
 
   template <int LIK, bool LAST>
@@ -452,14 +489,15 @@ struct MfmaLayer {
       TileIn ti;
       f4 acc[NT];
       load_tile_safe(ti, cx, tile * 16, n, q);
+      f2 xg[4];
       gemm1(ti.xa, acc);
-      pointwise<LIK, LAST, false>(acc, ti.yv, cx, mc, tile * 16, n, q);
-      gemm2(acc, ti.xb);
+      pointwise<LIK, LAST, false>(acc, ti.yv, ti.xb, xg, cx, mc, tile * 16, n, q);
+      gemm2(acc, xg);
     }
   }
 
   // this wave's partial sums -> its LDS slot, indexed by canonical parameter number; the factor
-  // w2[c] left out of delta is applied here
+  // 4 w2[c] left out of the GEMM2 operand is applied here
   __device__ __forceinline__ void write_partials(float* slot, const float* s_w) {
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
     static_assert(D1 % 16 != 0, "db2 rides in the first padded hidden unit");
@@ -472,16 +510,16 @@ struct MfmaLayer {
         for (int j = 0; j < 4; ++j) {
           const int c = 16 * t + 4 * q + j;
           if (c < D1) {
-            const float v = dacc[t][u][j] * s_w[oW2 + c];
+            const float v = dacc[t][u][j] * (4.0f * s_w[oW2 + c]);
             if (f < D0) slot[f * D1 + c] = v;
             else if (f == D0) slot[oB1 + c] = v;
           } else if (c == D1 && f == D0) {
-            slot[oB2] = dacc[t][u][j];  // sum of g over this wave's rows
+            slot[oB2] = 4.0f * dacc[t][u][j];  // sum of g over this wave's rows
           }
         }
       }
-      // dw2: sum the four row groups q in a fixed order
-      float v = dw2acc[t];
+      // dw2 = sum_rows g h = 2 sum_rows g s - sum_rows g; the four row groups q in a fixed order
+      float v = __builtin_fmaf(2.0f, dw2s[t], -gacc);
       v += __shfl_xor(v, 16);
       v += __shfl_xor(v, 32);
       const int c = 16 * t + n;
@@ -529,6 +567,7 @@ struct FfmaLayer {
     float yv;
   };
 
+  template <int LIK>
   __device__ __forceinline__ void load_weights(const float* s_w, const ModelConsts&) {
     const int lane = threadIdx.x & 63, cc = lane & 7;
 #pragma unroll
@@ -685,6 +724,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   __shared__ float s_w[P_AL];
   __shared__ __align__(16) float s_slots[W][SLOT];
   __shared__ double s_red[W];
+  __shared__ unsigned long long s_hash[W];
   __shared__ int s_flag;
 
   // ---- which chain group, which rank inside it ----
@@ -773,6 +813,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   }
   const int n_outer = trans ? a.n_trans : 1;
   double dl_total = 0.0;
+  unsigned long long hacc = 0;  // state hash, see fold_hash
 
   for (int it = 0; it < n_outer && ok; ++it) {
     const uint32_t t = (uint32_t)(t0 + it);
@@ -810,7 +851,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       }
       __syncthreads();
       BNN_PHASE(0)  // update + sync
-      layer.load_weights(s_w, mc);
+      layer.template load_weights<LIK>(s_w, mc);
       layer.zero_acc();
       BNN_PHASE(1)  // operand fetch from LDS
       const bool last = s == a.L - 1;
@@ -873,15 +914,13 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
             const float* src = grp_part + 4 * col;
             for (int r0 = part; r0 < a.G; r0 += 8 * H) {
               f4 t8[8];
+              const float* p8[8];
 #pragma unroll
-              for (int k = 0; k < 8; ++k) {
-                const int r = r0 + H * k;
-                if (r < a.G) ld_agent4_issue(t8[k], src + (size_t)r * SLOT);
-                else t8[k] = f4{0.f, 0.f, 0.f, 0.f};
-              }
-              wait_agent4x8(t8);
+              for (int k = 0; k < 8; ++k) p8[k] = src + (size_t)min(r0 + H * k, a.G - 1) * SLOT;
+              ld_agent4x8(t8, p8);
 #pragma unroll
-              for (int k = 0; k < 8; ++k) v += t8[k];
+              for (int k = 0; k < 8; ++k)
+                if (r0 + H * k < a.G) v += t8[k];  // wave-uniform condition
             }
             // rows 0 .. H-1 of s_slots are free: stage 1 read them before the barrier
             *reinterpret_cast<f4*>(&s_slots[part][4 * col]) = v;
@@ -925,15 +964,13 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
           f4 v = {0.f, 0.f, 0.f, 0.f};
           for (int r0 = rl; r0 < a.G; r0 += 8 * RL) {
             f4 t8[8];
+            const float* p8[8];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-              const int r = r0 + RL * k;
-              if (r < a.G) ld_agent4_issue(t8[k], src + (size_t)r * SLOT);
-              else t8[k] = f4{0.f, 0.f, 0.f, 0.f};
-            }
-            wait_agent4x8(t8);
+            for (int k = 0; k < 8; ++k) p8[k] = src + (size_t)min(r0 + RL * k, a.G - 1) * SLOT;
+            ld_agent4x8(t8, p8);
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v += t8[k];
+            for (int k = 0; k < 8; ++k)
+              if (r0 + RL * k < a.G) v += t8[k];
           }
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -1033,6 +1070,10 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         const float adj = lmin < a.log_target ? a.dec_adj : a.inc_adj;
         eps = eps + eps * adj;
       }
+      // what this workgroup holds after the transition goes into its state hash
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) hacc = fold_hash(hacc, wc[i], gc[i]);
+      hacc = fold_hash(hacc, la, eps) + (unsigned long long)nacc;
       if (rank == 0) {
         // ---- sample store (main.h:277-283) and traces ----
         if ((int)t >= a.burn_in && (int)t - a.burn_in < a.n_samples) {
@@ -1062,6 +1103,13 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   }
 #undef BNN_PHASE
   if (!ok) return;
+  if (a.rank_hash) {
+    if (!trans) {
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) hacc = fold_hash(fold_hash(hacc, w[i], g[i]), m[i], eps);
+    }
+    publish_hash(hacc, s_hash, W, a.rank_hash + lin, rank == a.debug_perturb_hash_rank);
+  }
   // ---- write back ----
   if (rank == 0) {
     if (trans) {

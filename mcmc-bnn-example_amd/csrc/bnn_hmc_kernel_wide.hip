@@ -314,6 +314,7 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
   float* s_g = s_m + P_AL;        // gradient at s_w
   float* s_red = s_g + P_AL;      // workgroup partial record (SLOT floats, the last four hold a double)
   __shared__ double s_wsum[W];
+  __shared__ unsigned long long s_hash[W];
   __shared__ int s_flag;
 
   int lin = blockIdx.x;
@@ -379,6 +380,7 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
   bool ok = true;
   const int n_outer = trans ? a.n_trans : 1;
   double dl_total = 0.0;
+  unsigned long long hacc = 0;  // state hash, see fold_hash
 
   for (int it = 0; it < n_outer && ok; ++it) {
     const uint32_t t = (uint32_t)(t0 + it);
@@ -438,14 +440,13 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
         const float* src = grp_part + 4 * col;
         for (int r0 = 0; r0 < a.G; r0 += 8) {
           f4 t8[8];
+          const float* p8[8];
 #pragma unroll
-          for (int k = 0; k < 8; ++k) {
-            if (r0 + k < a.G) ld_agent4_issue(t8[k], src + (size_t)(r0 + k) * SLOT);
-            else t8[k] = f4{0.f, 0.f, 0.f, 0.f};
-          }
-          wait_agent4x8(t8);
+          for (int k = 0; k < 8; ++k) p8[k] = src + (size_t)min(r0 + k, a.G - 1) * SLOT;
+          ld_agent4x8(t8, p8);
 #pragma unroll
-          for (int k = 0; k < 8; ++k) v += t8[k];
+          for (int k = 0; k < 8; ++k)
+            if (r0 + k < a.G) v += t8[k];
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -506,6 +507,9 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
         const float adj = lmin < a.log_target ? a.dec_adj : a.inc_adj;
         eps = eps + eps * adj;
       }
+      // what this workgroup holds after the transition goes into its state hash
+      for (int p = tid; p < P; p += T) hacc = fold_hash(hacc, wc[p], gc[p]);
+      hacc = fold_hash(hacc, la, eps) + (unsigned long long)nacc;
       if (rank == 0) {
         // ---- sample store (main.h:277-283) and traces ----
         if ((int)t >= a.burn_in && (int)t - a.burn_in < a.n_samples) {
@@ -522,6 +526,11 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
   }
 
   if (!ok) return;
+  if (a.rank_hash) {
+    if (!trans)
+      for (int p = tid; p < P; p += T) hacc = fold_hash(fold_hash(hacc, s_w[p], s_g[p]), s_m[p], eps);
+    publish_hash(hacc, s_hash, W, a.rank_hash + lin, rank == a.debug_perturb_hash_rank);
+  }
   if (rank == 0) {
     if (trans) {
       for (int p = tid; p < P; p += T) {

@@ -45,6 +45,36 @@ __device__ __forceinline__ double shfl_xor_d(double v, int mask) {
   return bits_to_double(((uint64_t)hi << 32) | lo);
 }
 
+__device__ __forceinline__ unsigned long long shfl_xor_u64(unsigned long long b, int mask) {
+  const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)b, mask);
+  const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(b >> 32), mask);
+  return ((unsigned long long)hi << 32) | lo;
+}
+
+// State hash of a workgroup.  Every workgroup of a chain group integrates the same parameters from
+// the same exchanged gradients and must hold the same bits; each folds what it holds into a 64-bit
+// value per thread (fold_hash), the values of a workgroup are added up when the kernel ends
+// (publish_hash) and the host compares the workgroups of a group.  A workgroup that ever read a
+// stale partial record ends with a different hash.
+__device__ __forceinline__ unsigned long long fold_hash(unsigned long long h, float a, float b) {
+  return mix64(h ^ (((unsigned long long)__builtin_bit_cast(uint32_t, a) << 32) |
+                    __builtin_bit_cast(uint32_t, b)));
+}
+// s_tmp: one slot per wave.  Contains two workgroup barriers: call from uniform control flow.
+__device__ __forceinline__ void publish_hash(unsigned long long h, unsigned long long* s_tmp, int n_waves,
+                                             unsigned long long* dst, bool perturb) {
+#pragma unroll
+  for (int msk = 1; msk < 64; msk <<= 1) h += shfl_xor_u64(h, msk);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) s_tmp[threadIdx.x >> 6] = h;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long tot = 0;
+    for (int wv = 0; wv < n_waves; ++wv) tot += s_tmp[wv];
+    *dst = perturb ? tot ^ 1ull : tot;
+  }
+}
+
 // activation of the hidden layer, include/mcmc/kernel_helpers.h:34-42:
 // tanh(x) = 2 sigmoid(2x) - 1 with e^(-2x) = 2^(x * -2/ln 2); identity below the cutoff
 __device__ __forceinline__ float tanh_fwd(float x) {
@@ -89,17 +119,27 @@ __device__ __forceinline__ float ld_agent(const float* p) {
 __device__ __forceinline__ void st_agent(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// 16-byte agent-scope load, issued without waiting: up to eight of them are collected with
-// wait_agent4x8 (the compiler neither reorders nor waits for loads issued from inline assembly)
-__device__ __forceinline__ void ld_agent4_issue(f4& d, const float* p) {
-  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(d) : "v"(p) : "memory");
-}
-__device__ __forceinline__ void wait_agent4x8(f4 (&t)[8]) {
-  asm volatile("s_waitcnt vmcnt(0)"
-               : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]),
-                 "+v"(t[7])
-               :
-               : "memory");
+// Eight 16-byte agent-scope loads in flight at once, collected before the statement ends: the loads
+// and the wait form ONE assembly statement, so the compiler sees the eight results as defined only
+// once they have landed (it may spill or copy them afterwards like any other value).  The results are
+// early-clobber: a returning load must not land in a register that still holds the address of a load
+// not yet issued.  Every address must be valid; callers clamp out-of-range records to a valid one and
+// discard the value.
+__device__ __forceinline__ void ld_agent4x8(f4 (&t)[8], const float* const (&p)[8]) {
+  asm volatile(
+      "global_load_dwordx4 %0, %8, off sc1\n\t"
+      "global_load_dwordx4 %1, %9, off sc1\n\t"
+      "global_load_dwordx4 %2, %10, off sc1\n\t"
+      "global_load_dwordx4 %3, %11, off sc1\n\t"
+      "global_load_dwordx4 %4, %12, off sc1\n\t"
+      "global_load_dwordx4 %5, %13, off sc1\n\t"
+      "global_load_dwordx4 %6, %14, off sc1\n\t"
+      "global_load_dwordx4 %7, %15, off sc1\n\t"
+      "s_waitcnt vmcnt(0)"
+      : "=&v"(t[0]), "=&v"(t[1]), "=&v"(t[2]), "=&v"(t[3]), "=&v"(t[4]), "=&v"(t[5]), "=&v"(t[6]),
+        "=&v"(t[7])
+      : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
+      : "memory");
 }
 
 // ------------------------------------------------------------------------------------------------

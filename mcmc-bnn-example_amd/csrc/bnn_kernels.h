@@ -21,6 +21,10 @@ hipError_t launch_hmc_kernel(const void* kernel, const KArgs& args, int workgrou
 // small kernels
 hipError_t launch_fill_u32(unsigned* p, size_t n, unsigned v, hipStream_t stream);
 hipError_t launch_fill_f32(float* p, size_t n, float v, hipStream_t stream);
+// compares the state hashes the workgroups of the last trajectory launch reported (see
+// compare_hashes_kernel); status words as described there
+hipError_t launch_compare_hashes(const unsigned long long* h, int wgs, int G, unsigned* status,
+                                 hipStream_t stream);
 hipError_t launch_sample_momentum(uint32_t seed, uint32_t chain_id, uint32_t transition, int n,
                                   float* a, float* b, hipStream_t stream);
 hipError_t launch_log_acpt(int n_loss, int n_mom, const float* prev_loss, const float* new_loss,

@@ -271,12 +271,25 @@ void eval_f32_range(const orc_model& m, const Consts& c, const Layout& L, const 
   }
 }
 
+// Rows are cut into fixed chunks of ROW_CHUNK rows (whatever the number of threads); each chunk is
+// summed on its own in block order and the chunk sums are added in chunk order, so the result does
+// not depend on how many threads ran.
+constexpr int ROW_CHUNK = 64 * ROW_BLOCK;
+
 void eval_f32(const orc_model& m, const float* X, const float* y, const float* w, float* ell,
               float* prior, float* grad, float* yhat) {
   Consts c(m);
   Layout L(m.d0, m.d1);
-  std::vector<double> gacc(L.P, 0.0);
-  eval_f32_range(m, c, L, X, y, w, 0, m.n, ell, gacc.data(), yhat);
+  const int n_chunks = (m.n + ROW_CHUNK - 1) / ROW_CHUNK;
+  std::vector<double> gacc((size_t)std::max(n_chunks, 1) * L.P, 0.0);
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static) if (n_chunks > 1)
+#endif
+  for (int ch = 0; ch < n_chunks; ++ch)
+    eval_f32_range(m, c, L, X, y, w, ch * ROW_CHUNK, std::min(m.n, (ch + 1) * ROW_CHUNK), ell,
+                   gacc.data() + (size_t)ch * L.P, yhat);
+  for (int ch = 1; ch < n_chunks; ++ch)
+    for (int p = 0; p < L.P; ++p) gacc[p] += gacc[(size_t)ch * L.P + p];
   for (int p = 0; p < L.P; ++p) {
     float lp, gp;
     prior_terms(c, w[p], &lp, &gp);
@@ -342,9 +355,20 @@ inline void leapfrog_update(float& w, float& mom, float g_prev, float eps, int m
   w = fmaf(eps, mom, w);
 }
 
+bool g_cut_short = true;  // see orc_set_cut_short
+
 }  // namespace
 
 extern "C" {
+
+void orc_set_threads(int threads) {
+#ifdef _OPENMP
+  if (threads > 0) omp_set_num_threads(threads);
+#else
+  (void)threads;
+#endif
+}
+void orc_set_cut_short(int on) { g_cut_short = on != 0; }
 
 int orc_num_params(int d0, int d1) { return Layout(d0, d1).P; }
 
@@ -417,6 +441,20 @@ void orc_mcmc_step(const orc_model* m, const float* X, const float* y, const flo
   for (int s = 0; s < L; ++s) {
     // ffma.h:408 (first launch: MOM_CORRECTION 2), 414-419 (middle), 420-426 (last: OUTPUT_LOSS)
     for (int p = 0; p < P; ++p) leapfrog_update(w[p], mom[p], g[p], eps, s == 0 ? 2 : 1);
+    // A position that has left the finite numbers never comes back (inf + x is inf or NaN), its
+    // log-prior is -inf or NaN, so the log accept ratio of this trajectory is -inf or NaN whatever
+    // the remaining steps do: the transition rejects and counts as -inf for the adaptation.  The
+    // remaining steps are skipped and every output is NaN.
+    bool finite = true;
+    for (int p = 0; p < P; ++p) finite = finite && std::isfinite(w[p]);
+    if (!finite && g_cut_short) {
+      const float nan = std::numeric_limits<float>::quiet_NaN();
+      std::fill(w.begin(), w.end(), nan);
+      std::fill(mom.begin(), mom.end(), nan);
+      std::fill(g.begin(), g.end(), nan);
+      std::fill(loss_values, loss_values + m->n + P, nan);
+      break;
+    }
     bool last = (s == L - 1);
     eval_f32(*m, X, y, w.data(), last ? loss_values : nullptr,
              last ? loss_values + m->n : nullptr, gn.data(), nullptr);
@@ -453,25 +491,31 @@ float orc_adapt_eps(const orc_hmc* h, float eps, float log_acpt) {
   return eps + eps * adj;
 }
 
-int orc_run_chain(const orc_model* m, const orc_hmc* h, const float* X, const float* y,
-                  float* samples, float* log_acpt_trace, int* accept_trace, float* eps_trace,
-                  float* final_w, float* final_eps) {
+// main.h:117-293 from a given state: position w0 (NULL = zeros, main.h:166-183), step size eps0 and
+// the index t0 of the first transition (which selects the RNG counters and the sample slots).
+static int run_chain_impl(const orc_model* m, const orc_hmc* h, const float* X, const float* y,
+                          const float* w0, float eps0, int t0, int n_trans, float* samples,
+                          float* log_acpt_trace, int* accept_trace, float* eps_trace, float* final_w,
+                          float* final_eps) {
   const int P = orc_num_params(m->d0, m->d1);
   const int n = m->n;
-  // main.h:166-183: all state starts at zero
   std::vector<float> w(P, 0.0f), mom(P, 0.0f), g(P, 0.0f);
   std::vector<float> w_next(P), mom_next(P), g_cur(P), loss(n + P), prev_loss(n + P), prev_g(P),
       prev_w(P, 0.0f), mom0(P);
-  float eps = h->eps0;
-  // bootstrap main.h:191-202: one step from the all-zero state is a no-op update followed by an
-  // evaluation at w = 0
+  if (w0) {
+    std::copy(w0, w0 + P, w.begin());
+    std::copy(w0, w0 + P, prev_w.begin());
+  }
+  float eps = eps0;
+  // bootstrap main.h:191-202: with zero momentum and zero gradient the update is a no-op, so one
+  // step evaluates the log-posterior rows and the gradient at the start
   orc_mcmc_step(m, X, y, w.data(), mom.data(), g.data(), eps, 1, w_next.data(), mom_next.data(),
                 g_cur.data(), loss.data());
   prev_g = g_cur;
   prev_loss = loss;
   int n_acc = 0;
-  const int total = h->burn_in + h->n_samples;
-  for (int step = 0; step < total; ++step) {
+  for (int i = 0; i < n_trans; ++i) {
+    const int step = t0 + i;
     orc_momentum(h->seed, h->chain_id, (uint32_t)step, P, mom0.data());  // main.h:207-216
     // main.h:218-223: trajectory from (prev_w, mom0, prev_g)
     orc_mcmc_step(m, X, y, prev_w.data(), mom0.data(), prev_g.data(), eps, h->leapfrog_steps,
@@ -486,16 +530,31 @@ int orc_run_chain(const orc_model* m, const orc_hmc* h, const float* X, const fl
       prev_loss = loss;
       ++n_acc;
     }  // else main.h:254-265: the saved state stays
-    if (log_acpt_trace) log_acpt_trace[step] = la;
-    if (accept_trace) accept_trace[step] = acc;
+    if (log_acpt_trace) log_acpt_trace[i] = la;
+    if (accept_trace) accept_trace[i] = acc;
     if (step < h->adapt_steps) eps = orc_adapt_eps(h, eps, la);  // main.h:267-276
-    if (eps_trace) eps_trace[step] = eps;
-    if (step >= h->burn_in && samples)  // main.h:277-283
+    if (eps_trace) eps_trace[i] = eps;
+    if (step >= h->burn_in && step - h->burn_in < h->n_samples && samples)  // main.h:277-283
       std::memcpy(samples + (size_t)(step - h->burn_in) * P, prev_w.data(), sizeof(float) * P);
   }
   if (final_w) std::memcpy(final_w, prev_w.data(), sizeof(float) * P);
   if (final_eps) *final_eps = eps;
   return n_acc;
+}
+
+int orc_run_chain(const orc_model* m, const orc_hmc* h, const float* X, const float* y,
+                  float* samples, float* log_acpt_trace, int* accept_trace, float* eps_trace,
+                  float* final_w, float* final_eps) {
+  return run_chain_impl(m, h, X, y, nullptr, h->eps0, 0, h->burn_in + h->n_samples, samples,
+                        log_acpt_trace, accept_trace, eps_trace, final_w, final_eps);
+}
+
+int orc_run_chain_from(const orc_model* m, const orc_hmc* h, const float* X, const float* y,
+                       const float* w0, float eps0, int t0, int n_trans, float* samples,
+                       float* log_acpt_trace, int* accept_trace, float* eps_trace, float* final_w,
+                       float* final_eps) {
+  return run_chain_impl(m, h, X, y, w0, eps0, t0, n_trans, samples, log_acpt_trace, accept_trace,
+                        eps_trace, final_w, final_eps);
 }
 
 void orc_final_loss(const orc_model* m, const float* X, const float* y, const float* samples,

@@ -28,6 +28,9 @@
  *   orc_log_acpt              H_prev - H_new recomputed from scratch in float64          pinned
  *   orc_accept / orc_adapt    exhaustive small table; closed-form eps product            pinned
  *   orc_run_chain             composition of the above + sample-store invariants         pinned
+ *   orc_run_chain_from        equals the tail of orc_run_chain from its own saved state  pinned
+ *   row-parallel evaluation   same bits with 1, 3 and 8 threads                          pinned
+ *   cut-short trajectories    same decisions / step sizes as full-length NaN ones        pinned
  *   bit-level outputs of the reference's CUDA kernels (atomic order, ex2.approx / rcp.approx ulps,
  *   cub reduction trees, thrust/libstdc++ RNG streams): the reference ships no test vectors and
  *   cannot be built here                                                        parity unpinned
@@ -71,6 +74,12 @@ typedef struct orc_hmc {
 } orc_hmc;
 
 int orc_num_params(int d0, int d1);
+/* number of OpenMP threads the row-parallel evaluations use from now on (results do not depend on it) */
+void orc_set_threads(int threads);
+/* 0: orc_mcmc_step integrates every step even after the position has become non-finite (as the
+ * reference does); 1 (default): it stops there.  Decisions and step sizes are the same either way;
+ * the switch exists so that a test can show it. */
+void orc_set_cut_short(int on);
 
 /* ---- RNG (build-defined; replaces main.h:207-216 and main.h:235-239) ---- */
 void orc_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
@@ -109,7 +118,9 @@ void orc_eval_f64(const orc_model* m, const float* X, const float* y, const doub
 /* ---- the step operator: L fused leapfrog steps                           (ffma.h:395-427) ----
  * in : w_prev, mom_prev, grad_prev (= full gradient at w_prev), eps, L >= 1
  * out: w_next, mom_next (lacking the final half step), grad_cur (full gradient at w_next),
- *      loss_values[n + P] (per-row log-lik then per-parameter log-prior at w_next) */
+ *      loss_values[n + P] (per-row log-lik then per-parameter log-prior at w_next)
+ * A trajectory whose position leaves the finite numbers is cut short there and returns NaN in every
+ * output (the transition would reject whatever the remaining steps did). */
 void orc_mcmc_step(const orc_model* m, const float* X, const float* y, const float* w_prev,
                    const float* mom_prev, const float* grad_prev, float eps, int L, float* w_next,
                    float* mom_next, float* grad_cur, float* loss_values);
@@ -128,6 +139,15 @@ float orc_adapt_eps(const orc_hmc* h, float eps, float log_acpt);
 int orc_run_chain(const orc_model* m, const orc_hmc* h, const float* X, const float* y,
                   float* samples, float* log_acpt_trace, int* accept_trace, float* eps_trace,
                   float* final_w, float* final_eps);
+
+/* The same from a given state: position w0 (P floats, NULL = zeros), step size eps0, first
+ * transition index t0 (selects the RNG counters, the adaptation window and the sample slots), for
+ * n_trans transitions.  Traces have length n_trans; samples[h->n_samples][P] receives the rows whose
+ * transition index falls in [burn_in, burn_in + n_samples). */
+int orc_run_chain_from(const orc_model* m, const orc_hmc* h, const float* X, const float* y,
+                       const float* w0, float eps0, int t0, int n_trans, float* samples,
+                       float* log_acpt_trace, int* accept_trace, float* eps_trace, float* final_w,
+                       float* final_eps);
 
 /* mean log-lik / log-prior over samples                                    (main.h:78-115) */
 void orc_final_loss(const orc_model* m, const float* X, const float* y, const float* samples,

@@ -74,7 +74,14 @@ class Oracle:
         L.orc_adapt_eps.restype = C.c_float
         L.orc_adapt_eps.argtypes = [C.POINTER(Hmc), C.c_float, C.c_float]
         L.orc_run_chain.restype = C.c_int
+        L.orc_run_chain_from.restype = C.c_int
         L.orc_bench_grad_evals.restype = C.c_double
+
+    def set_threads(self, threads):
+        self.lib.orc_set_threads(C.c_int(threads))
+
+    def set_cut_short(self, on):
+        self.lib.orc_set_cut_short(C.c_int(1 if on else 0))
 
     def num_params(self, d0, d1):
         return self.lib.orc_num_params(d0, d1)
@@ -209,6 +216,25 @@ class Oracle:
                                        acc.ctypes.data_as(C.POINTER(C.c_int)), _fp(eps), _fp(fw),
                                        C.byref(fe))
         return dict(samples=samples, log_acpt=la, accept=acc, eps=eps, final_w=fw,
+                    final_eps=fe.value, n_accept=n_acc)
+
+    def run_chain_from(self, m, h, X, y, w0, eps0, t0, n_trans):
+        """n_trans transitions from position w0 (None = zeros), step size eps0, transition index t0."""
+        P = self.num_params(m.d0, m.d1)
+        X = np.ascontiguousarray(X, np.float32)
+        y = np.ascontiguousarray(y, np.float32)
+        w0p = None if w0 is None else _fp(np.ascontiguousarray(w0, np.float32))
+        samples = np.full((max(h.n_samples, 1), P), np.nan, np.float32)
+        la = np.empty(n_trans, np.float32)
+        acc = np.empty(n_trans, np.int32)
+        eps = np.empty(n_trans, np.float32)
+        fw = np.empty(P, np.float32)
+        fe = C.c_float()
+        n_acc = self.lib.orc_run_chain_from(C.byref(m), C.byref(h), _fp(X), _fp(y), w0p, C.c_float(eps0),
+                                            C.c_int(t0), C.c_int(n_trans), _fp(samples), _fp(la),
+                                            acc.ctypes.data_as(C.POINTER(C.c_int)), _fp(eps), _fp(fw),
+                                            C.byref(fe))
+        return dict(samples=samples[:h.n_samples], log_acpt=la, accept=acc, eps=eps, final_w=fw,
                     final_eps=fe.value, n_accept=n_acc)
 
     def final_loss(self, m, X, y, samples):

@@ -485,6 +485,61 @@ def test_run_chain_bookkeeping(orc):
     assert out["final_eps"] == out["eps"][h.adapt_steps - 1] == out["eps"][-1]
 
 
+def test_run_chain_from_a_saved_state_is_the_tail_of_the_whole_chain(orc):
+    n = 96
+    m, X, y, _ = _case(orc, n, "gauss", seed=13)
+    h = ob.Hmc(8, 12, 20, 12, 1e-2, 0.2, 0.1, 0.01, 77, 5)
+    whole = orc.run_chain(m, h, X, y)
+    for cut in (5, 12, 19):    # inside the adaptation window, at its end, among the kept samples
+        head = orc.run_chain_from(m, h, X, y, None, h.eps0, 0, cut)
+        assert head["accept"].tobytes() == whole["accept"][:cut].tobytes()
+        tail = orc.run_chain_from(m, h, X, y, head["final_w"], head["final_eps"], cut, 32 - cut)
+        assert tail["accept"].tobytes() == whole["accept"][cut:].tobytes()
+        assert tail["eps"].tobytes() == whole["eps"][cut:].tobytes()
+        assert tail["log_acpt"].tobytes() == whole["log_acpt"][cut:].tobytes()
+        first = max(cut, h.burn_in) - h.burn_in
+        assert tail["samples"][first:].tobytes() == whole["samples"][first:].tobytes()
+        assert tail["final_w"].tobytes() == whole["final_w"].tobytes()
+
+
+def test_row_parallel_evaluation_does_not_depend_on_the_thread_count(orc):
+    n = 5000   # five chunks of 1024 rows, the last one short
+    m, X, y, w = _case(orc, n, "t", seed=15)
+    outs = []
+    for threads in (1, 3, 8):
+        orc.set_threads(threads)
+        ell, prior, g, yh = orc.eval_f32(m, X, y, w)
+        outs.append(ell.tobytes() + prior.tobytes() + g.tobytes() + yh.tobytes())
+    orc.set_threads(8)
+    assert outs[0] == outs[1] == outs[2]
+    # and the chunked sum is the plain sum over rows: float64 gradient of the same model
+    _, _, g64 = orc.eval_f64(m, X, y, w.astype(np.float64))
+    np.testing.assert_allclose(g, g64, rtol=0, atol=2e-6 * np.abs(g64).max())
+
+
+def test_cut_short_trajectories_decide_like_full_length_ones(orc):
+    # the stiff Gaussian posterior with eps0 = 0.01 overflows within a few steps until the adaptation
+    # has shrunk the step size: integrating on through NaN (as the reference does) and stopping at the
+    # first non-finite position must give the same decisions and step sizes
+    n = 512
+    m, X, y, _ = _case(orc, n, "gauss", seed=16)
+    h = ob.Hmc(30, 60, 4, 60, 1e-2, 0.2, 0.1, 0.01, 3, 0)
+    try:
+        orc.set_cut_short(False)
+        full = orc.run_chain(m, h, X, y)
+    finally:
+        orc.set_cut_short(True)
+    cut = orc.run_chain(m, h, X, y)
+    assert not np.isfinite(full["log_acpt"][0]) and full["accept"][0] == 0
+    assert 0 < full["accept"].sum()                      # the chain does get going
+    assert cut["accept"].tobytes() == full["accept"].tobytes()
+    assert cut["eps"].tobytes() == full["eps"].tobytes()
+    assert cut["samples"].tobytes() == full["samples"].tobytes()
+    finite = np.isfinite(full["log_acpt"])
+    assert np.array_equal(finite, np.isfinite(cut["log_acpt"]))
+    assert cut["log_acpt"][finite].tobytes() == full["log_acpt"][finite].tobytes()
+
+
 def test_final_loss_is_mean_over_samples(orc):
     n = 50
     m, X, y, w = _case(orc, n, "t", seed=14)
