@@ -64,6 +64,8 @@ typedef struct bnnhmc_hmc {
   float decrement;    /* 0.1  */
   float increment;    /* 0.01 */
   uint32_t seed;      /* RNG key word 0; key word 1 is the global chain index */
+  uint32_t chain_id_base; /* global index of this sampler's chain 0 (default 0): a sampler that  */
+                      /* holds a slice of a larger job draws the streams the whole job would  */
 } bnnhmc_hmc;
 
 /* How the work is laid over the GPU.  Zero in a field selects the default. */

@@ -29,7 +29,8 @@ class Model(C.Structure):
 class Hmc(C.Structure):
     _fields_ = [("leapfrog_steps", C.c_int), ("burn_in", C.c_int), ("n_samples", C.c_int),
                 ("adapt_steps", C.c_int), ("eps0", C.c_float), ("target_rate", C.c_float),
-                ("decrement", C.c_float), ("increment", C.c_float), ("seed", C.c_uint32)]
+                ("decrement", C.c_float), ("increment", C.c_float), ("seed", C.c_uint32),
+                ("chain_id_base", C.c_uint32)]
 
 
 class Launch(C.Structure):

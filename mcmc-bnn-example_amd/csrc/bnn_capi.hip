@@ -324,6 +324,10 @@ int debug_drop_rank() {
 // Test hook: BNNHMC_DEBUG_PERTURB_HASH=<rank> makes that rank of every chain group flip one bit of
 // the state hash it reports (its memory traffic and its results are untouched), so that the
 // comparison of the hashes fails.  Unset in normal use.
+int env_balance() {
+  const char* e = getenv("BNNHMC_BALANCE");
+  return e && *e ? atoi(e) : 1;
+}
 int debug_perturb_hash_rank() {
   const char* e = getenv("BNNHMC_DEBUG_PERTURB_HASH");
   return e && *e ? atoi(e) : -1;
@@ -482,6 +486,7 @@ KArgs base_args(const bnnhmc_sampler* s) {
   a.spin_limit = s->plan.spin_limit;
   a.debug_drop_rank = debug_drop_rank();
   a.debug_perturb_hash_rank = debug_perturb_hash_rank();
+  a.balance = env_balance();
   Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups);
   a.partials = w.partials;
   a.totals = w.totals;
@@ -562,6 +567,7 @@ void bnnhmc_default_hmc(bnnhmc_hmc* h) {
   h->decrement = 0.1f;
   h->increment = 0.01f;
   h->seed = 0;
+  h->chain_id_base = 0;
 }
 
 void bnnhmc_default_launch(bnnhmc_launch* l) {
@@ -729,6 +735,7 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
   a.spin_limit = plan.spin_limit;
   a.debug_drop_rank = debug_drop_rank();
   a.debug_perturb_hash_rank = debug_perturb_hash_rank();
+  a.balance = env_balance();
   Workspace w = carve_workspace(workspace, L.P, G, 1);
   a.partials = w.partials;
   a.totals = w.totals;
@@ -1008,6 +1015,7 @@ int bnnhmc_run(bnnhmc_sampler* s, int n_transitions) {
       a.tr_eps = s->tr_eps;
       a.trace_len = s->trace_len;
       a.seed = s->hmc.seed;
+      a.rng_id_base = s->hmc.chain_id_base;
       a.debug_phase = s->debug_phase;
       int rc = launch_and_count(s, a, groups);
       if (rc) return rc;

@@ -82,6 +82,7 @@ struct KArgs {
   int chains_per_window;
   int fixed_window; // >= 0: every group reads this window
   int xcd_map;      // 1: blockIdx is spread round-robin over 8 XCDs, keep a group inside one XCD
+  int balance;      // 1: the two waves of a SIMD keep pace through wave priorities (prefetched loop)
   // ---- what to do ----
   int mode;
   int L;            // leapfrog steps per trajectory
@@ -123,6 +124,7 @@ struct KArgs {
   float* tr_eps;
   int trace_len;
   uint32_t seed;
+  uint32_t rng_id_base;  // RNG key word 1 of chain c is rng_id_base + c
   // ---- cross-workgroup exchange ----
   float* partials;     // [group][2][G][slot]
   float* totals;       // [group][slot]: reduced gradient, two-phase reduction only

@@ -72,13 +72,19 @@ struct MfmaLayer {
   // affine in s or products of s, and the constants move into per-step operands (one VALU
   // instruction less per hidden value and row).
   float w1b[KS][NT];   // W1_aug scaled by -2/ln 2: GEMM1 yields the exp2 argument t of the activation
-  float w2g[NT];       // -2 w2[c] k with k = 1/scale^2 (Gaussian: the layer-2 dot yields the per-row
-                       // loss gradient g directly) or 1/scale (Student-t: it yields the scaled residual)
-  float y_k;           // k in lane n == 0, else 0
-  float y_0;           // (sum_c w2[c] - b2) k in lane n == 0, else 0: the constant part of the dot
-  f4 dacc[NT][2];      // sum over rows of s (1 - s) g x_aug: dW1_aug^T / (4 w2[c])
-  float dw2s[NT];      // sum over rows of g s
-  float gacc;          // sum over rows of g, added in the order of dw2s: dw2 = 2 dw2s - gacc is then
+  float w2g[NT];       // -2 w2[c] k2: the layer-2 dot yields r = (y - yhat - b2) k2, where k2 is the power
+                       // of two next to k = 1/scale^2 (Gaussian: r k / k2 is the per-row loss gradient)
+                       // or k = 1/scale (Student-t: r k / k2 is the scaled residual).  A power of two
+                       // keeps the coefficients exact: the dot cancels from terms of size |w2| k to a
+                       // residual thousands of times smaller, and a rounding error in a coefficient
+                       // would be the same in every row and add up over the rows instead of averaging out
+  float y_k;           // k2 in lane n == 0, else 0
+  float y_0;           // the constant part of the dot, (sum_c w2[c] - b2) k2, computed in double and
+                       // split over lanes n == 0 (leading part) and n == 1 (remainder)
+  float ratio;         // k / k2 (exact)
+  f4 dacc[NT][2];      // sum over rows of s (1 - s) g' x_aug, g' = g k2 / k (Gaussian) or g (Student-t)
+  float dw2s[NT];      // sum over rows of g' s
+  float gacc;          // sum over rows of g', added in the order of dw2s: dw2 = 2 dw2s - gacc is then
                        // exactly zero where every s is 1/2 (all weights zero, the reference's start)
   double dl;
 
@@ -94,7 +100,12 @@ struct MfmaLayer {
   __device__ __forceinline__ void load_weights(const float* s_w, const ModelConsts& mc) {
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
     const float k = LIK == 1 ? mc.scale_recp * mc.scale_recp : mc.scale_recp;
-    float w2sum = 0.0f;
+    // the power of two next to k, and its reciprocal
+    const uint32_t k2_bits = (__builtin_bit_cast(uint32_t, k) + 0x00400000u) & 0x7F800000u;
+    const float k2 = __builtin_bit_cast(float, k2_bits);
+    ratio = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
+        int, k * __builtin_bit_cast(float, 0x7F000000u - k2_bits))));
+    double w2sum = 0.0;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int c = 16 * t + n;
@@ -109,12 +120,16 @@ struct MfmaLayer {
         w1b[s][t] = cv ? v * kExp2Scale : 0.0f;
       }
       const float w2c = cv ? s_w[oW2 + cc] : 0.0f;
-      w2sum += w2c;
-      w2g[t] = -2.0f * w2c * k;
+      w2sum += (double)w2c;
+      w2g[t] = -2.0f * w2c * k2;
     }
-    w2sum = row16_allreduce(w2sum);  // sum over all hidden units, the same bits in every lane
-    y_k = n == 0 ? k : 0.0f;
-    y_0 = n == 0 ? (w2sum - s_w[oB2]) * k : 0.0f;
+    // sum over all hidden units in double, the same bits in every lane of a row of 16
+#pragma unroll
+    for (int msk = 1; msk < 16; msk <<= 1) w2sum += shfl_xor_d(w2sum, msk);
+    const double c0 = (w2sum - (double)s_w[oB2]) * (double)k2;
+    const float c0_hi = (float)c0, c0_lo = (float)(c0 - (double)c0_hi);
+    y_k = n == 0 ? k2 : 0.0f;
+    y_0 = n == 0 ? c0_hi : (n == 1 ? c0_lo : 0.0f);
   }
 
   __device__ __forceinline__ void zero_acc() {
@@ -204,17 +219,17 @@ struct MfmaLayer {
       const float r = row16_allreduce(yh[j]);
       float gj, diff;
       if (LIK == 0) {
-        diff = r;
+        diff = r * ratio;
         gj = diff * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(diff, diff, mc.df));
       } else {
-        gj = r;
+        gj = r;  // the factor k / k2 is applied to the sums, once per step
       }
       const bool valid = FULL || (row0 + 4 * q + j < cx.n);
       gj = valid ? gj : 0.0f;  // mcmc_step_ffma.h:301
       g[j] = gj;
       if (LAST) {
         if (n == 0 && valid) {
-          if (LIK == 1) diff = r * mc.scale;
+          if (LIK == 1) diff = r * (ratio * mc.scale);
           const int row = row0 + 4 * q + j;
           const float lv = lik_value<LIK>(mc, diff);
           const float prev = cx.ell_prev ? cx.ell_prev[row] : 0.0f;
@@ -443,7 +458,11 @@ struct MfmaLayer {
       f2 xg[4];
       gemm1(xa, acc);
       pointwise<LIK, LAST, true>(acc, t.yv, t.xb, xg, cx, mc, tile * 16, n, q);
+      // keep the stages apart: left to itself the scheduler may feed each GEMM2 operand to its
+      // MFMAs the moment it is computed, which puts two wait states in front of every other MFMA
+      __builtin_amdgcn_sched_barrier(0);
       gemm2(acc, xg);
+      __builtin_amdgcn_sched_barrier(0);
     };
     TileRaw A, B, C;
     preset(A);
@@ -451,8 +470,14 @@ struct MfmaLayer {
     preset(C);
     issue(A);
     issue(B);
-    // steady state: three tiles per trip, every issue and every wait unconditional
+    // steady state: three tiles per trip, every issue and every wait unconditional.
+    // Two waves share a SIMD, and the matrix and vector instructions of both go through one FP32
+    // pipe: it stays busy only while both waves have work (each fills the dependency stalls of the
+    // other).  The hardware favours the older wave, which would finish its tiles long before the
+    // younger one and leave it to run alone, stalls exposed.  So every trip a wave publishes its
+    // tile count in LDS, reads its partner's, and takes the higher priority while it is behind.
     int i = tb;
+    const bool balance = cx.progress != nullptr;
     for (; i + 3 <= te; i += 3) {
       issue(C);
       wait_tile<14>(A);
@@ -463,7 +488,21 @@ struct MfmaLayer {
       issue(B);
       wait_tile<14>(C);
       compute(C, i + 2);
+      if (balance) {
+        // all operands are wave-uniform: the registers live only across these three instructions
+        const unsigned my_slot = (unsigned)(size_t)(cx.progress + cx.wave);  // LDS byte addresses
+        const unsigned other_slot = (unsigned)(size_t)(cx.progress + cx.partner);
+        const int done = i + 3 - tb;
+        int other;
+        asm volatile("ds_write_b32 %1, %2\n\tds_read_b32 %0, %3\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(other)
+                     : "v"(my_slot), "v"(done), "v"(other_slot)
+                     : "memory");
+        if (__builtin_amdgcn_readfirstlane(other) > done) __builtin_amdgcn_s_setprio(2);
+        else __builtin_amdgcn_s_setprio(0);
+      }
     }
+    if (balance) __builtin_amdgcn_s_setprio(0);
     // no register of a set may be used or reused before its last load has landed
     wait_tile<0>(A);
     wait_tile<0>(B);
@@ -496,11 +535,14 @@ struct MfmaLayer {
     }
   }
 
-  // this wave's partial sums -> its LDS slot, indexed by canonical parameter number; the factor
-  // 4 w2[c] left out of the GEMM2 operand is applied here
+  // this wave's partial sums -> its LDS slot, indexed by canonical parameter number; the factors
+  // 4 w2[c] left out of the GEMM2 operand and k / k2 left out of g are applied here
+  template <int LIK>
   __device__ __forceinline__ void write_partials(float* slot, const float* s_w) {
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
     static_assert(D1 % 16 != 0, "db2 rides in the first padded hidden unit");
+    const float gr = LIK == 1 ? ratio : 1.0f;
+    const float gr4 = 4.0f * gr;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -510,16 +552,16 @@ struct MfmaLayer {
         for (int j = 0; j < 4; ++j) {
           const int c = 16 * t + 4 * q + j;
           if (c < D1) {
-            const float v = dacc[t][u][j] * (4.0f * s_w[oW2 + c]);
+            const float v = dacc[t][u][j] * (gr4 * s_w[oW2 + c]);
             if (f < D0) slot[f * D1 + c] = v;
             else if (f == D0) slot[oB1 + c] = v;
           } else if (c == D1 && f == D0) {
-            slot[oB2] = 4.0f * dacc[t][u][j];  // sum of g over this wave's rows
+            slot[oB2] = gr4 * dacc[t][u][j];  // sum of g over this wave's rows
           }
         }
       }
       // dw2 = sum_rows g h = 2 sum_rows g s - sum_rows g; the four row groups q in a fixed order
-      float v = __builtin_fmaf(2.0f, dw2s[t], -gacc);
+      float v = __builtin_fmaf(2.0f, dw2s[t], -gacc) * gr;
       v += __shfl_xor(v, 16);
       v += __shfl_xor(v, 32);
       const int c = 16 * t + n;
@@ -679,6 +721,7 @@ struct FfmaLayer {
     return v;
   }
 
+  template <int LIK>
   __device__ __forceinline__ void write_partials(float* slot, const float*) {
     const int lane = threadIdx.x & 63, cc = lane & 7, rg = lane >> 3;
 #pragma unroll
@@ -713,6 +756,18 @@ struct FfmaLayer {
 // ------------------------------------------------------------------------------------------------
 // the kernel
 // ------------------------------------------------------------------------------------------------
+// Kernel arguments that are needed once per transition or once per launch are not kept in registers
+// across the step loop (they would be spilled into lanes of vector registers, which the tile loop has
+// none to spare of): COLD(field) reads the field from the kernel-argument segment where it is used.
+// The empty assembly statement makes the pointer opaque, so that the load stays where it is written.
+__device__ __forceinline__ const __attribute__((address_space(4))) KArgs* cold_args() {
+  const __attribute__((address_space(4))) KArgs* p =
+      (const __attribute__((address_space(4))) KArgs*)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(p));
+  return p;
+}
+#define COLD(field) (cold_args()->field)
+
 template <class Layer, int LIK, int T>
 __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   constexpr int W = T / 64;
@@ -725,6 +780,12 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   __shared__ __align__(16) float s_slots[W][SLOT];
   __shared__ double s_red[W];
   __shared__ unsigned long long s_hash[W];
+  __shared__ int s_progress[W];
+  // kept out of registers while a trajectory runs (a thread only ever touches the entries of the
+  // parameters it owns, so no barrier guards them): the accepted position and its gradient, the
+  // start momentum of the running transition, and the thread's state hash
+  __shared__ float s_wc[PPT * T], s_gc[PPT * T], s_m0[PPT * T];
+  __shared__ unsigned long long s_hacc[T];
   __shared__ int s_flag;
 
   // ---- which chain group, which rank inside it ----
@@ -757,6 +818,10 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   }
   cx.ell_prev = nullptr;
   cx.ell_new = nullptr;
+  // waves w and w + W / 2 sit on the same SIMD (waves are dealt to the four SIMDs in turn)
+  cx.progress = (a.balance && W == 8) ? s_progress : nullptr;
+  cx.wave = wave;
+  cx.partner = wave ^ (W / 2);
 
   const ModelConsts mc = a.mc;
   float* part_base = a.partials + (size_t)group * 2 * a.G * SLOT;
@@ -765,18 +830,19 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   int buf = 0;
 
   // ---- parameters owned by this thread: p = tid + i T ----
-  float w[PPT], m[PPT], g[PPT], wc[PPT], gc[PPT], m0[PPT];
+  float w[PPT], m[PPT], g[PPT];
   float eps;
   int t0 = 0, sel = 0, nacc = 0;
   const bool trans = a.mode == MODE_TRANSITIONS;
 #pragma unroll
   for (int i = 0; i < PPT; ++i) {
     const int p = tid + i * T;
-    w[i] = m[i] = g[i] = wc[i] = gc[i] = m0[i] = 0.0f;
+    w[i] = m[i] = g[i] = 0.0f;
+    s_wc[tid + i * T] = s_gc[tid + i * T] = s_m0[tid + i * T] = 0.0f;
     if (p < P) {
       if (trans) {
-        wc[i] = a.st_w[(size_t)chain * a.st_stride + p];
-        gc[i] = a.st_g[(size_t)chain * a.st_stride + p];
+        s_wc[p] = a.st_w[(size_t)chain * a.st_stride + p];
+        s_gc[p] = a.st_g[(size_t)chain * a.st_stride + p];
       } else {
         const size_t o = (size_t)group * a.in_stride + p;
         w[i] = a.w_in ? a.w_in[o] : 0.0f;
@@ -813,7 +879,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   }
   const int n_outer = trans ? a.n_trans : 1;
   double dl_total = 0.0;
-  unsigned long long hacc = 0;  // state hash, see fold_hash
+  s_hacc[tid] = 0;  // state hash, see fold_hash
 
   for (int it = 0; it < n_outer && ok; ++it) {
     const uint32_t t = (uint32_t)(t0 + it);
@@ -825,16 +891,16 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       for (int i = 0; i < PPT; ++i) {
         const int p = tid + i * T;
         if (p < P) {
-          m0[i] = rng_normal(a.seed, (uint32_t)chain, STREAM_MOMENTUM, t, (uint64_t)p);
-          m[i] = m0[i];
-          w[i] = wc[i];
-          g[i] = gc[i];
+          m[i] = rng_normal(COLD(seed), (uint32_t)chain + COLD(rng_id_base), STREAM_MOMENTUM, t, (uint64_t)p);
+          s_m0[p] = m[i];
+          w[i] = s_wc[p];
+          g[i] = s_gc[p];
         }
       }
-      ell_cur = (sel ? a.ell1 : a.ell0) + (size_t)chain * a.ell_stride;
-      ell_prop = (sel ? a.ell0 : a.ell1) + (size_t)chain * a.ell_stride;
+      ell_cur = (sel ? COLD(ell1) : COLD(ell0)) + (size_t)chain * COLD(ell_stride);
+      ell_prop = (sel ? COLD(ell0) : COLD(ell1)) + (size_t)chain * COLD(ell_stride);
     } else {
-      ell_prop = a.ell_out ? a.ell_out + (size_t)group * a.ell_stride : nullptr;
+      ell_prop = COLD(ell_out) ? COLD(ell_out) + (size_t)group * COLD(ell_stride) : nullptr;
     }
 
     for (int s = 0; s < a.L && ok; ++s) {
@@ -849,6 +915,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
           s_w[p] = w[i];
         }
       }
+      if ((tid & 63) == 0) s_progress[wave] = 0;
       __syncthreads();
       BNN_PHASE(0)  // update + sync
       layer.template load_weights<LIK>(s_w, mc);
@@ -863,7 +930,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         layer.template run_tiles<LIK, false>(cx, mc);
       }
       BNN_PHASE(2)  // tile loop
-      layer.write_partials(s_slots[wave], s_w);
+      layer.template write_partials<LIK>(s_slots[wave], s_w);
       __syncthreads();
       BNN_PHASE(3)  // wave partials -> LDS + sync
       // ---- stage 1: fixed-order sum over this workgroup's waves -> global partial record ----
@@ -1035,9 +1102,10 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       for (int i = 0; i < PPT; ++i) {
         const int p = tid + i * T;
         if (p < P) {
-          const float dp = prior_logp(mc, w[i]) - prior_logp(mc, wc[i]);
+          const float dp = prior_logp(mc, w[i]) - prior_logp(mc, s_wc[p]);
           const float nm = __builtin_fmaf(eps * 0.5f, g[i], m[i]);  // final half kick
-          float kt = m0[i] * m0[i];
+          const float m0 = s_m0[p];
+          float kt = m0 * m0;
           kt = __builtin_fmaf(-nm, nm, kt);
           part += (double)dp + (double)(0.5f * kt);
         }
@@ -1052,42 +1120,45 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       for (int wv = 0; wv < W; ++wv) tot += s_red[wv];
       const float la = (float)tot;
       // ---- Metropolis decision (main.h:235-265) ----
-      const float lu = rng_log_uniform(a.seed, (uint32_t)chain, t);
+      const float lu = rng_log_uniform(COLD(seed), (uint32_t)chain + COLD(rng_id_base), t);
       const bool acc = lu < la;
       if (acc) {
 #pragma unroll
         for (int i = 0; i < PPT; ++i) {
-          wc[i] = w[i];
-          gc[i] = g[i];
+          s_wc[tid + i * T] = w[i];
+          s_gc[tid + i * T] = g[i];
         }
         sel ^= 1;
         ++nacc;
       }
       // ---- step-size adaptation (main.h:267-276); a non-finite ratio counts as minus infinity ----
-      if ((int)t < a.adapt_steps) {
+      if ((int)t < COLD(adapt_steps)) {
         const float laf = (la == la) ? la : -__builtin_inff();
         const float lmin = laf < 0.0f ? laf : 0.0f;
-        const float adj = lmin < a.log_target ? a.dec_adj : a.inc_adj;
+        const float adj = lmin < COLD(log_target) ? COLD(dec_adj) : COLD(inc_adj);
         eps = eps + eps * adj;
       }
       // what this workgroup holds after the transition goes into its state hash
+      {
+        unsigned long long hacc = s_hacc[tid];
 #pragma unroll
-      for (int i = 0; i < PPT; ++i) hacc = fold_hash(hacc, wc[i], gc[i]);
-      hacc = fold_hash(hacc, la, eps) + (unsigned long long)nacc;
+        for (int i = 0; i < PPT; ++i) hacc = fold_hash(hacc, s_wc[tid + i * T], s_gc[tid + i * T]);
+        s_hacc[tid] = fold_hash(hacc, la, eps) + (unsigned long long)nacc;
+      }
       if (rank == 0) {
         // ---- sample store (main.h:277-283) and traces ----
-        if ((int)t >= a.burn_in && (int)t - a.burn_in < a.n_samples) {
-          float* dst = a.samples + ((size_t)chain * a.n_samples + ((int)t - a.burn_in)) * P;
+        if ((int)t >= COLD(burn_in) && (int)t - COLD(burn_in) < COLD(n_samples)) {
+          float* dst = COLD(samples) + ((size_t)chain * COLD(n_samples) + ((int)t - COLD(burn_in))) * P;
 #pragma unroll
           for (int i = 0; i < PPT; ++i) {
             const int p = tid + i * T;
-            if (p < P) dst[p] = wc[i];
+            if (p < P) dst[p] = s_wc[p];
           }
         }
-        if (tid == 0 && (int)t < a.trace_len) {
-          a.tr_log_acpt[(size_t)chain * a.trace_len + t] = la;
-          a.tr_accept[(size_t)chain * a.trace_len + t] = acc ? 1 : 0;
-          a.tr_eps[(size_t)chain * a.trace_len + t] = eps;
+        if (tid == 0 && (int)t < COLD(trace_len)) {
+          COLD(tr_log_acpt)[(size_t)chain * COLD(trace_len) + t] = la;
+          COLD(tr_accept)[(size_t)chain * COLD(trace_len) + t] = acc ? 1 : 0;
+          COLD(tr_eps)[(size_t)chain * COLD(trace_len) + t] = eps;
         }
       }
     }
@@ -1096,19 +1167,20 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   if (prof && tid == 0) {
     BNN_PHASE(7)  // transition epilogue
 #pragma unroll
-    for (int k = 0; k < 8; ++k) a.debug_phase[(size_t)blockIdx.x * 10 + k] = ph[k];
+    for (int k = 0; k < 8; ++k) COLD(debug_phase)[(size_t)blockIdx.x * 10 + k] = ph[k];
     // shader-clock ticks and 100 MHz real-time ticks of the whole launch: their ratio is the clock
-    a.debug_phase[(size_t)blockIdx.x * 10 + 8] = __builtin_readcyclecounter() - clk0;
-    a.debug_phase[(size_t)blockIdx.x * 10 + 9] = __builtin_amdgcn_s_memrealtime() - rt0;
+    COLD(debug_phase)[(size_t)blockIdx.x * 10 + 8] = __builtin_readcyclecounter() - clk0;
+    COLD(debug_phase)[(size_t)blockIdx.x * 10 + 9] = __builtin_amdgcn_s_memrealtime() - rt0;
   }
 #undef BNN_PHASE
   if (!ok) return;
-  if (a.rank_hash) {
+  if (COLD(rank_hash)) {
+    unsigned long long hacc = s_hacc[tid];
     if (!trans) {
 #pragma unroll
       for (int i = 0; i < PPT; ++i) hacc = fold_hash(fold_hash(hacc, w[i], g[i]), m[i], eps);
     }
-    publish_hash(hacc, s_hash, W, a.rank_hash + lin, rank == a.debug_perturb_hash_rank);
+    publish_hash(hacc, s_hash, W, COLD(rank_hash) + lin, rank == COLD(debug_perturb_hash_rank));
   }
   // ---- write back ----
   if (rank == 0) {
@@ -1117,15 +1189,15 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       for (int i = 0; i < PPT; ++i) {
         const int p = tid + i * T;
         if (p < P) {
-          a.st_w[(size_t)chain * a.st_stride + p] = wc[i];
-          a.st_g[(size_t)chain * a.st_stride + p] = gc[i];
+          COLD(st_w)[(size_t)chain * COLD(st_stride) + p] = s_wc[p];
+          COLD(st_g)[(size_t)chain * COLD(st_stride) + p] = s_gc[p];
         }
       }
       if (tid == 0) {
-        a.st_eps[chain] = eps;
-        a.st_t[chain] = t0 + a.n_trans;
-        a.st_sel[chain] = sel;
-        a.st_nacc[chain] = nacc;
+        COLD(st_eps)[chain] = eps;
+        COLD(st_t)[chain] = t0 + COLD(n_trans);
+        COLD(st_sel)[chain] = sel;
+        COLD(st_nacc)[chain] = nacc;
       }
     } else {
       double psum = 0.0;
@@ -1133,17 +1205,17 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       for (int i = 0; i < PPT; ++i) {
         const int p = tid + i * T;
         if (p < P) {
-          const size_t o = (size_t)group * a.out_stride + p;
+          const size_t o = (size_t)group * COLD(out_stride) + p;
           const float lp = prior_logp(mc, w[i]);
-          if (a.w_out) a.w_out[o] = w[i];
-          if (a.m_out) a.m_out[o] = m[i];
-          if (a.g_out) a.g_out[o] = g[i];
-          if (a.g_zero) a.g_zero[o] = 0.0f;
-          if (a.prior_out) a.prior_out[o] = lp;
+          if (COLD(w_out)) COLD(w_out)[o] = w[i];
+          if (COLD(m_out)) COLD(m_out)[o] = m[i];
+          if (COLD(g_out)) COLD(g_out)[o] = g[i];
+          if (COLD(g_zero)) COLD(g_zero)[o] = 0.0f;
+          if (COLD(prior_out)) COLD(prior_out)[o] = lp;
           psum += (double)lp;
         }
       }
-      if (a.sums_out) {
+      if (COLD(sums_out)) {
 #pragma unroll
         for (int msk = 1; msk < 64; msk <<= 1) psum += shfl_xor_d(psum, msk);
         __syncthreads();
@@ -1153,13 +1225,15 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
           double tot = 0.0;
 #pragma unroll
           for (int wv = 0; wv < W; ++wv) tot += s_red[wv];
-          a.sums_out[(size_t)group * 2 + 0] = dl_total;
-          a.sums_out[(size_t)group * 2 + 1] = tot;
+          COLD(sums_out)[(size_t)group * 2 + 0] = dl_total;
+          COLD(sums_out)[(size_t)group * 2 + 1] = tot;
         }
       }
     }
   }
 }
+
+#undef COLD
 
 // ------------------------------------------------------------------------------------------------
 // host-side launcher

@@ -390,7 +390,7 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
       // momentum resampling (main.h:207-216); the start state is the last accepted one.  Every
       // thread owns the parameters p = tid, tid + T, ... throughout.
       for (int p = tid; p < P; p += T) {
-        const float z = rng_normal(a.seed, (uint32_t)chain, STREAM_MOMENTUM, t, (uint64_t)p);
+        const float z = rng_normal(a.seed, (uint32_t)chain + a.rng_id_base, STREAM_MOMENTUM, t, (uint64_t)p);
         m0[p] = z;
         s_m[p] = z;
         s_w[p] = wc[p];
@@ -490,7 +490,7 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
       for (int wv = 0; wv < W; ++wv) tot += s_wsum[wv];
       const float la = (float)tot;
       // ---- Metropolis decision (main.h:235-265) ----
-      const float lu = rng_log_uniform(a.seed, (uint32_t)chain, t);
+      const float lu = rng_log_uniform(a.seed, (uint32_t)chain + a.rng_id_base, t);
       const bool acc = lu < la;
       if (acc) {
         for (int p = tid; p < P; p += T) {

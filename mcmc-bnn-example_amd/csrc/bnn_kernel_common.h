@@ -153,6 +153,8 @@ struct StepCtx {
   bool x_vec_ok, y_vec_ok;
   const float* ell_prev;  // last step only: rows of the current state (null = zeros)
   float* ell_new;         // last step only: where to store this state's rows (null = skip)
+  int* progress;          // LDS, one word per wave: tiles done in this step (null = no balancing)
+  int wave, partner;      // this wave and the wave it shares a SIMD with
 };
 
 // ------------------------------------------------------------------------------------------------

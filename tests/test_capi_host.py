@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol(pkg, lib):
 
 def test_struct_layouts_match_header(pkg):
     assert C.sizeof(pkg.Model) == 4 * 4 + 3 * 8
-    assert C.sizeof(pkg.Hmc) == 4 * 4 + 4 * 4 + 4
+    assert C.sizeof(pkg.Hmc) == 4 * 4 + 4 * 4 + 2 * 4
     assert C.sizeof(pkg.Launch) == 7 * 4
 
 

@@ -1,0 +1,306 @@
+"""GPU parity at the sizes the benchmark configurations state: 58368 rows, 1000 leapfrog steps per
+transition, 200 windows, 1600 kept samples.  The CPU oracle evaluates rows in parallel, so a
+58368-row x 1000-step trajectory costs it about a second on the GPU box's 16 cores."""
+import sys
+import time
+
+import numpy as np
+import pytest
+
+import orc_binding as ob
+from hipmem import DevBuf, synchronize
+
+pytestmark = pytest.mark.gpu
+
+D0, D1, P = 22, 40, 961
+N_FULL, L_FULL = 58368, 1000
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+# ------------------------------------------------------------------------------------------------
+# configs[0] as stated: one window, one chain, Gaussian likelihood sigma = 0.01, prior N(0, 0.1^2),
+# 58368 rows, 1000 leapfrog steps, the reference's eps0 = 0.01 and adaptation over the burn-in
+# ------------------------------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def config0_chain(pkg, lib, orc):
+    """Runs the first 100 transitions (the burn-in) of configs[0] on the GPU, keeps the sampler open
+    for the tests that continue it, and returns what they need."""
+    model = lib.default_model(n=N_FULL, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
+    om = ob.Model(D0, D1, N_FULL, ob.LIK_GAUSSIAN, 0.01, 0.0, 0.1)
+    hmc = lib.default_hmc(leapfrog_steps=L_FULL, burn_in=100, n_samples=100, eps0=0.01, seed=0)
+    oh = ob.Hmc(L_FULL, 100, 100, 100, 0.01, 0.2, 0.1, 0.01, 0, 0)
+    s = lib.create(model, hmc, lib.default_launch(), 1, 1)   # one chain: widened to all 256 CUs
+    s.generate_window(0, teacher_scale=0.1, noise_sigma=0.01)
+    X, y = s.get_window_data(0)
+    s.init_chains(None)
+    say("configs[0]: 100 burn-in transitions of 1000 leapfrog steps on the GPU")
+    s.run(100)
+    out = dict(s=s, model=model, om=om, oh=oh, X=X, y=y, traces=s.get_traces(0), state=s.get_chain_state(0))
+    yield out
+    s.close()
+
+
+def test_first_50_transitions_at_full_size(config0_chain, orc):
+    """north-star: identical accept/reject decisions over the first 50 transitions given the same RNG
+    stream.  With eps0 = 0.01 this posterior (curvature about n / sigma^2) makes every one of them
+    diverge: all reject, and the step-size trace must equal the oracle's bit for bit."""
+    c = config0_chain
+    t0 = time.time()
+    ref = orc.run_chain_from(c["om"], c["oh"], c["X"], c["y"], None, 0.01, 0, 50)
+    say("oracle: 50 transitions in %.1f s" % (time.time() - t0))
+    tr = c["traces"]
+    assert np.array_equal(tr["accept"][:50], ref["accept"])
+    assert tr["eps"][:50].tobytes() == ref["eps"].tobytes()
+    assert ref["accept"].sum() == 0                       # documented: all 50 are divergent
+    assert np.all(~np.isfinite(tr["log_acpt"][:50]) | (tr["log_acpt"][:50] < -1e6))
+    # the adaptation does arrive: later burn-in transitions accept
+    assert tr["accept"][50:100].sum() > 10
+    assert 5e-6 < c["state"]["eps"] < 1e-4
+
+
+def test_20_transitions_from_the_adapted_state_at_full_size(config0_chain, orc):
+    """The second leg: from the state the burn-in ends in (step size about 2e-5, weights of order
+    10), 20 transitions of 1000 leapfrog steps on the GPU and on the oracle, same RNG counters.
+
+    The log accept ratio is a sum over 58368 rows at the end of a 1000-step trajectory; FP32 rounding
+    differences of the gradient (1e-7 relative) grow along it, and the two implementations were
+    measured to differ by up to 0.062 in it.  Decisions must therefore agree wherever the uniform is
+    further than MARGIN = 0.15 from the oracle's ratio; how many transitions fall inside the margin is
+    reported, and at most two of the 20 may disagree in all."""
+    MARGIN = 0.15
+    c = config0_chain
+    s, st = c["s"], c["state"]
+    assert st["transitions_done"] == 100
+    s.run(20)
+    tr = s.get_traces(0)
+    t0 = time.time()
+    ref = orc.run_chain_from(c["om"], c["oh"], c["X"], c["y"], st["w"], st["eps"], 100, 20)
+    say("oracle: 20 full-length transitions in %.1f s" % (time.time() - t0))
+    lu = np.array([orc.log_uniform(0, 0, 100 + k) for k in range(20)])
+    la_gpu, la_ref = tr["log_acpt"][100:120], ref["log_acpt"]
+    acc_gpu, acc_ref = tr["accept"][100:120], ref["accept"]
+    clear = np.abs(lu - la_ref) > MARGIN
+    say("adapted leg: %d of 20 transitions inside the margin; max |log alpha gpu - oracle| = %.4f; "
+        "accepted gpu %d, oracle %d" % ((~clear).sum(), np.abs(la_gpu - la_ref).max(), acc_gpu.sum(),
+                                         acc_ref.sum()))
+    assert np.all(np.isfinite(la_gpu)) and np.all(np.isfinite(la_ref))
+    assert np.array_equal(acc_gpu[clear], acc_ref[clear])
+    assert clear.sum() >= 12, "too few transitions outside the margin to say anything"
+    assert (acc_gpu != acc_ref).sum() <= 2
+    assert np.abs(la_gpu - la_ref).max() < MARGIN
+    assert 0 < acc_ref.sum() < 20 or acc_ref.sum() == 20      # an adapted chain accepts most of them
+    # the step size no longer changes after the burn-in
+    assert np.all(tr["eps"][100:120] == np.float32(st["eps"]))
+
+
+# ------------------------------------------------------------------------------------------------
+# saturated hidden units: where the sampler spends its time
+# ------------------------------------------------------------------------------------------------
+def _saturated_bound(g_hip, g32, g64, what):
+    scale = float(np.abs(g64).max())
+    err_hip = float(np.abs(g_hip.astype(np.float64) - g64).max())
+    err_ref = float(np.abs(g32.astype(np.float64) - g64).max())
+    say("%s: |hip - f64| = %.3e, |f32 oracle - f64| = %.3e, max |g| = %.3e" % (what, err_hip, err_ref, scale))
+    assert err_hip <= 2.0 * err_ref + 1e-5 * scale, what
+
+
+@pytest.mark.parametrize("layer", ["mfma", "ffma"])
+def test_gradient_in_the_saturated_regime(config0_chain, pkg, lib, orc, layer):
+    """After the burn-in the weights are of order 10 and a third of the hidden pre-activations lie
+    beyond |x| > 4: 1 - tanh^2 cancels and no FP32 evaluation (the reference's formulation included)
+    reaches 1e-5.  The meaningful bound there: the HIP gradient may be at most twice as far from the
+    FP64 gradient as the FP32 restatement of the reference is, plus 1e-5 of the gradient scale."""
+    c = config0_chain
+    w = c["state"]["w"]
+    pre = c["X"] @ w[:D0 * D1].reshape(D0, D1) + w[D0 * D1:D0 * D1 + D1]
+    assert np.abs(w).max() > 5 and (np.abs(pre) > 4).mean() > 0.15, "the state is not saturated"
+    launch = lib.default_launch(layer=pkg.LAYER_MFMA if layer == "mfma" else pkg.LAYER_FFMA, cus_per_chain=32)
+    s = lib.create(c["model"], lib.default_hmc(seed=0), launch, 1, 1)
+    s.set_window_data(0, c["X"], c["y"])
+    ell, prior, g = s.eval(0, w)
+    s.close()
+    ell32, prior32, g32, _ = orc.eval_f32(c["om"], c["X"], c["y"], w)
+    ell64, _, g64 = orc.eval_f64(c["om"], c["X"], c["y"], w.astype(np.float64))
+    _saturated_bound(g, g32, g64, "22->40->1 %s gradient" % layer)
+    _saturated_bound(ell, ell32, ell64, "22->40->1 %s log-likelihood rows" % layer)
+    assert prior.tobytes() == prior32.tobytes()
+
+
+def test_gradient_in_the_saturated_regime_wide(pkg, lib, orc):
+    n = 8192
+    model = lib.default_model(d0=64, d1=128, n=n, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
+    om = ob.Model(64, 128, n, ob.LIK_GAUSSIAN, 0.01, 0.0, 0.1)
+    s = lib.create(model, lib.default_hmc(seed=4), lib.default_launch(cus_per_chain=16), 1, 1)
+    th = s.generate_window(0, teacher_scale=0.1, noise_sigma=0.01)
+    X, y = s.get_window_data(0)
+    w = (6.0 * th).astype(np.float32)                     # pre-activations of order 5
+    pre = X @ w[:64 * 128].reshape(64, 128) + w[64 * 128:64 * 128 + 128]
+    assert (np.abs(pre) > 4).mean() > 0.3
+    ell, prior, g = s.eval(0, w)
+    s.close()
+    ell32, _, g32, _ = orc.eval_f32(om, X, y, w)
+    ell64, _, g64 = orc.eval_f64(om, X, y, w.astype(np.float64))
+    _saturated_bound(g, g32, g64, "64->128->1 gradient")
+    _saturated_bound(ell, ell32, ell64, "64->128->1 log-likelihood rows")
+
+
+# ------------------------------------------------------------------------------------------------
+# configs[3]: 1600 kept samples (RNG counters, traces and sample slots past 900 transitions)
+# ------------------------------------------------------------------------------------------------
+def test_1600_samples_at_reduced_size(pkg, lib, orc):
+    n, L, burn, keep = 160, 4, 100, 1600
+    model = lib.default_model(n=n, lik_scale=1.0, prior_scale=0.5)
+    om = ob.Model(D0, D1, n, ob.LIK_STUDENT_T, 1.0, 2.2, 0.5)
+    hmc = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=0.01, seed=1600)
+    s = lib.create(model, hmc, lib.default_launch(cus_per_chain=2, transitions_per_launch=64), 1, 1)
+    s.generate_window(0, teacher_scale=0.3, noise_sigma=1.0)
+    X, y = s.get_window_data(0)
+    s.init_chains(None)
+    s.run(burn + keep)
+    samples, tr, st = s.get_samples(0), s.get_traces(0), s.get_chain_state(0)
+    l1, l2, fl = s.final_loss(0)
+    s.close()
+    ref = orc.run_chain(om, ob.Hmc(L, burn, keep, burn, 0.01, 0.2, 0.1, 0.01, 1600, 0), X, y)
+    T = burn + keep
+    assert samples.shape == (keep, P) and len(tr["accept"]) == T and st["transitions_done"] == T
+    lu = np.array([orc.log_uniform(1600, 0, t) for t in range(T)])
+    say("1600 samples: accept rate %.3f, smallest |log u - log alpha| %.2e" % (
+        ref["accept"].mean(), np.abs(lu - ref["log_acpt"]).min()))
+    assert np.array_equal(tr["accept"], ref["accept"])           # all 1700 decisions
+    assert tr["eps"].tobytes() == ref["eps"].tobytes()
+    assert 0.3 < ref["accept"].mean() < 1.0 and (ref["accept"][burn:] == 0).sum() > 10
+    scale = max(1.0, float(np.abs(ref["samples"]).max()))
+    np.testing.assert_allclose(samples[800:], ref["samples"][800:], rtol=0, atol=5e-4 * scale)
+    np.testing.assert_allclose(samples[:800], ref["samples"][:800], rtol=0, atol=5e-4 * scale)
+    np.testing.assert_allclose(st["w"], ref["final_w"], rtol=0, atol=5e-4 * scale)
+    assert st["n_accepted"] == ref["n_accept"]
+    for t in range(burn + 1, T):                                  # rejected transitions repeat the row
+        if not tr["accept"][t]:
+            assert np.array_equal(samples[t - burn], samples[t - burn - 1])
+    o1, o2, ofl = orc.final_loss(om, X, y, samples)
+    assert l1 == pytest.approx(o1, rel=1e-5) and l2 == pytest.approx(o2, rel=1e-6) and fl == pytest.approx(ofl, rel=1e-5)
+    # the momentum stream of the last transition, device == oracle bit for bit
+    a = DevBuf.full(P, np.nan)
+    lib.sample_momentum(1600, 0, T - 1, P, a.ptr, 0, 0)
+    synchronize()
+    assert a.numpy(P).tobytes() == orc.momentum(1600, 0, T - 1, P).tobytes()
+
+
+# ------------------------------------------------------------------------------------------------
+# configs[2] batching: 200 windows of 58368 rows as three batches of 64 (4 workgroups per chain) and
+# a last batch of 8 (widened to 32 workgroups per chain)
+# ------------------------------------------------------------------------------------------------
+def test_200_windows_are_batched_without_crosstalk(pkg, lib, orc):
+    # a step size small enough that trajectories from the all-zero start are accepted
+    L, burn, keep, eps0 = 50, 1, 1, 1e-6
+    model = lib.default_model(n=N_FULL, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
+    hmc = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=eps0, seed=0, adapt_steps=0)
+    say("200 windows: generating")
+    big = lib.create(model, hmc, lib.default_launch(), 200, 1)
+    for w in range(200):
+        big.generate_window(w, teacher_scale=0.1, noise_sigma=0.01)
+    big.init_chains(None)
+    say("200 windows: two transitions of every window")
+    big.run(burn + keep)
+    assert big.timing()["grad_evals"] == 200 * 2 * L
+    checks = {}
+    for chain in (0, 63, 64, 191, 192, 199):
+        checks[chain] = (big.get_samples(chain), big.get_traces(chain), big.get_chain_state(chain),
+                         big.get_window_data(chain) if chain in (0, 199) else None)
+        assert np.all(np.isfinite(checks[chain][0])) and checks[chain][2]["transitions_done"] == 2
+        assert checks[chain][2]["n_accepted"] >= 1 and np.abs(checks[chain][0]).max() > 0
+    big.close()
+    assert not np.array_equal(checks[63][0], checks[64][0])       # different windows, different chains
+    # chain 0 sat in a batch of 64 at 4 workgroups per chain, chain 199 in the tail batch of 8 at 32:
+    # each must equal, bit for bit, a sampler that holds only that window and is launched that way
+    for chain, G in ((0, 4), (199, 32)):
+        X, y = checks[chain][3]
+        h1 = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=eps0, seed=0,
+                             adapt_steps=0, chain_id_base=chain)
+        one = lib.create(model, h1, lib.default_launch(cus_per_chain=G), 1, 1)
+        one.set_window_data(0, X, y)
+        one.init_chains(None)
+        one.run(burn + keep)
+        assert one.get_samples(0).tobytes() == checks[chain][0].tobytes(), chain
+        tr1, trb = one.get_traces(0), checks[chain][1]
+        assert tr1["log_acpt"].tobytes() == trb["log_acpt"].tobytes(), chain
+        assert np.array_equal(tr1["accept"], trb["accept"])
+        st1, stb = one.get_chain_state(0), checks[chain][2]
+        assert st1["w"].tobytes() == stb["w"].tobytes() and st1["grad"].tobytes() == stb["grad"].tobytes()
+        one.close()
+    # and window 0's data is the recipe's: the oracle's generator gives the same bits
+    Xo, yo, _ = orc.gen_window(0, 0, N_FULL)
+    assert checks[0][3][0].tobytes() == Xo.tobytes() and checks[0][3][1].tobytes() == yo.tobytes()
+
+
+# ------------------------------------------------------------------------------------------------
+# the workgroups of a chain must hold the same state: checked after every launch
+# ------------------------------------------------------------------------------------------------
+def test_divergence_of_a_workgroup_is_reported(pkg, lib, orc, monkeypatch):
+    n = 4096
+    model = lib.default_model(n=n)
+    s = lib.create(model, lib.default_hmc(leapfrog_steps=5, burn_in=2, n_samples=2),
+                   lib.default_launch(cus_per_chain=4), 2, 1)
+    ths = [s.generate_window(w, teacher_scale=0.3, noise_sigma=5.0) for w in range(2)]
+    # one rank reports a hash with a flipped bit (its memory traffic and results are untouched)
+    monkeypatch.setenv("BNNHMC_DEBUG_PERTURB_HASH", "3")
+    with pytest.raises(pkg.BnnHmcError) as e:
+        s.eval(0, ths[0])
+    assert e.value.code == pkg.ERR_DIVERGED and "different state" in str(e.value)
+    with pytest.raises(pkg.BnnHmcError) as e:
+        s.init_chains(None)
+    assert e.value.code == pkg.ERR_DIVERGED
+    monkeypatch.delenv("BNNHMC_DEBUG_PERTURB_HASH")
+    s.init_chains(None)                                   # the sampler stays usable
+    s.run(2)
+    monkeypatch.setenv("BNNHMC_DEBUG_PERTURB_HASH", "1")
+    with pytest.raises(pkg.BnnHmcError) as e:
+        s.run(2)
+    assert e.value.code == pkg.ERR_DIVERGED
+    monkeypatch.delenv("BNNHMC_DEBUG_PERTURB_HASH")
+    s.close()
+    # the step operator reports it through bnnhmc_step_check
+    X, y, th = orc.gen_window(1, 0, n, teacher_scale=0.3, noise_sigma=5.0)
+    launch = lib.default_launch(cus_per_chain=8)
+    dev = DevBuf.from_numpy
+    dX, dy, dw, dm, dg = dev(X), dev(y), dev(th), dev(np.ones(P, np.float32)), dev(np.zeros(P, np.float32))
+    outs = [DevBuf.full(P, 0.0) for _ in range(4)]
+    dloss = DevBuf.full(n + P, 0.0)
+    wsb = lib.step_workspace_bytes(model, launch)
+    ws = DevBuf.full(wsb // 4 + 16, 0, np.int32)
+    for perturb, code in (("5", pkg.ERR_DIVERGED), (None, None)):
+        if perturb:
+            monkeypatch.setenv("BNNHMC_DEBUG_PERTURB_HASH", perturb)
+        lib.mcmc_step(model, launch, dX.ptr, dy.ptr, dw.ptr, outs[0].ptr, dm.ptr, outs[1].ptr, dg.ptr,
+                      outs[2].ptr, outs[3].ptr, dloss.ptr, ws.ptr, wsb, 0.01, 3, 0)
+        if code is None:
+            lib.step_check(model, launch, ws.ptr, 0)
+        else:
+            with pytest.raises(pkg.BnnHmcError) as e:
+                lib.step_check(model, launch, ws.ptr, 0)
+            assert e.value.code == code
+            monkeypatch.delenv("BNNHMC_DEBUG_PERTURB_HASH")
+
+
+def test_single_chain_on_256_workgroups_soak(pkg, lib, orc):
+    """One chain on every compute unit (the two-phase exchange across all eight XCDs), 200 000
+    leapfrog steps: any workgroup that ever read an incomplete partial record would end a launch with
+    a different state hash, which the call reports."""
+    model = lib.default_model(n=N_FULL, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
+    hmc = lib.default_hmc(leapfrog_steps=1000, burn_in=200, n_samples=0, eps0=2e-4, seed=7)
+    s = lib.create(model, hmc, lib.default_launch(cus_per_chain=256, transitions_per_launch=10), 1, 1)
+    s.generate_window(0, teacher_scale=0.1, noise_sigma=0.01)
+    s.init_chains(None)
+    t0 = time.time()
+    for k in range(4):
+        s.run(50)
+        say("soak: %d steps, %.1f s" % ((k + 1) * 50000, time.time() - t0))
+    st = s.get_chain_state(0)
+    assert st["transitions_done"] == 200 and bool(np.all(np.isfinite(st["w"])))
+    assert st["n_accepted"] > 20, st["n_accepted"]           # the adaptation got the chain going
+    assert s.timing()["workgroups"] == 256
+    s.close()
