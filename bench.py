@@ -1,14 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the HMC hot path on one MI355X.
 
-Workload (BASELINE.json configs[2]): independent windows of the 22->40->1 Bayesian MLP, full batch of
-58368 rows each (features ~ N(0,1), teacher-MLP targets + N(0, 0.01^2) noise, Gaussian likelihood,
-Gaussian weight prior), HMC with 1000 leapfrog steps per transition.  As many windows as are
-co-resident on the GPU form one batch; a "step" is one HMC transition (momentum resampling, 1000 fused
-leapfrog gradient evaluations, log accept ratio, Metropolis decision, adaptation, sample store) of
-every window of the batch.  The metric is leapfrog gradient evaluations per second; the minutes for
-200 windows x (100 burn-in + 800 samples) follow from it and are labelled as extrapolated unless
---full runs that whole job.
+Workload (BASELINE.json configs[2], the configuration the metric is quoted on): 200 independent windows
+of the 22->40->1 Bayesian MLP, full batch of 58368 rows each (features ~ N(0,1), teacher-MLP targets +
+N(0, 0.01^2) noise, Gaussian likelihood, Gaussian weight prior), one chain per window, HMC with 1000
+leapfrog steps per transition, all 200 windows resident in HBM (1.07 GB).  A "step" is one HMC transition
+(momentum resampling, 1000 fused leapfrog gradient evaluations, log accept ratio, Metropolis decision,
+sample store) of every one of the 200 windows: the library runs them as three batches of 64 chains at 4
+workgroups per chain and a last batch of 8 chains at 32 workgroups per chain.  The warm-up transitions
+are the burn-in (nothing stored), the timed ones store their samples.  The metric is leapfrog gradient
+evaluations per second; the minutes for 200 windows x (100 burn-in + 800 samples) are 900 steps plus the
+bootstrap evaluation, and --full runs that whole job.
 
 Prints ONE JSON line.  Inputs are resident in HBM before the timed region starts.
 """
@@ -28,10 +30,18 @@ WIDE_ROWS, WIDE_D0, WIDE_D1, WIDE_CHAINS = 4 * 58368, 64, 128, 4
 PEAK_TFLOPS = 157.3                         # MI355X dense FP32 matrix peak (v_mfma_f32_16x16x4_f32)
 EVALS_200x800 = 200 * (900 * 1000 + 1)      # 200 windows x ((100 + 800) transitions x 1000 steps + bootstrap)
 EVALS_200x1600 = 200 * (1700 * 1000 + 1)
-# HBM-side bytes per gradient evaluation of the MFMA trajectory kernel, from rocprofv3 FETCH_SIZE and
-# WRITE_SIZE scaled by a 1 GiB copy kernel (profiles/hmc_kernel_mfma_22x40_64windows.txt): one window's
-# X and y (5.37 MB) pass through L2 once per leapfrog step, plus the partial-gradient records.
-TRAFFIC_BYTES_PER_EVAL_MFMA = 1.7287e12 / 320000
+# HBM-side bytes per gradient evaluation of the trajectory kernels, measured with rocprofv3 FETCH_SIZE
+# and WRITE_SIZE scaled by a 1 GiB copy kernel: written by mcmc-bnn-example_amd/profile_summary.py
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(kernel_key):
+    """bytes per gradient evaluation of `kernel_key` from profiles/traffic.json, or None"""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            return float(json.load(f)[kernel_key]["bytes_per_grad_eval"])
+    except (OSError, KeyError, ValueError, TypeError):
+        return None
 
 
 def cpu_baseline(seconds, n_rows=N_ROWS, d0=D0, d1=D1):
@@ -61,18 +71,21 @@ def main():
     ap.add_argument("--wgs-per-cu", type=int, default=0)
     ap.add_argument("--threads", type=int, default=0)
     ap.add_argument("--pipeline", type=int, default=0)
-    ap.add_argument("--windows", type=int, default=0, help="0 = as many as are co-resident")
+    ap.add_argument("--windows", type=int, default=0,
+                    help="0 = 200 (the configuration the metric is quoted on); --shape wide: as many as are "
+                         "co-resident")
     ap.add_argument("--leapfrog", type=int, default=1000)
     ap.add_argument("--transitions-per-launch", type=int, default=5)
     ap.add_argument("--eps0", type=float, default=2e-5,
-                    help="initial leapfrog step size of the timed transitions: about what the adaptation "
-                         "reaches on this posterior; --full starts from the reference's 0.01 and adapts")
+                    help="leapfrog step size of the timed transitions: what the adaptation reaches on this "
+                         "posterior; --full starts from the reference's 0.01 and adapts")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="0 skips the CPU baseline")
     ap.add_argument("--shape", choices=["base", "wide"], default="base",
                     help="base = configs[2] (22->40->1, the metric's configuration); wide = configs[4] "
                          "(64->128->1, 233472 rows, 4 chains per window)")
     ap.add_argument("--full", action="store_true",
-                    help="run the whole 200 windows x (100 + 800) transitions job and time all of it")
+                    help="run the whole 200 windows x (100 + 800) transitions job from the all-zero start with "
+                         "the reference's adaptation and time all of it")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU (windows are independent: more GPUs would only run more windows "
@@ -107,18 +120,25 @@ def main():
     wgs_per_cu = 1 if wide or layer != pkg.LAYER_MFMA else launch.wgs_per_cu
     group = launch.cus_per_chain or 4
     resident = max(1, (cus * wgs_per_cu) // group)          # chains in flight
-    n_windows = 200 if args.full else (args.windows or max(1, resident // cpw))
+    n_windows = args.windows or (max(1, resident // cpw) if wide else 200)
     n_chains = n_windows * cpw
 
     model = lib.default_model(d0=d0, d1=d1, n=n_rows, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01,
                               prior_scale=0.1)
-    burn, keep = (100, 800) if args.full else (args.warmup + args.steps, 0)
-    hmc = lib.default_hmc(leapfrog_steps=args.leapfrog, burn_in=burn, n_samples=keep, seed=0)
+    if args.full:
+        burn, keep, adapt = 100, 800, 100
+    else:  # warm-up = burn-in (nothing stored), timed transitions store their samples; no adaptation
+        burn, keep, adapt = args.warmup, args.steps, 0
+    hmc = lib.default_hmc(leapfrog_steps=args.leapfrog, burn_in=burn, n_samples=keep, adapt_steps=adapt, seed=0)
     if not args.full:
         hmc.eps0 = args.eps0
     s = lib.create(model, hmc, launch, n_windows, cpw)
+    teachers = []
+    t_gen = time.perf_counter()
     for w in range(n_windows):
-        s.generate_window(w, teacher_scale=0.1, noise_sigma=0.01)  # untimed, like the reference's load
+        teachers.append(s.generate_window(w, teacher_scale=0.1, noise_sigma=0.01))  # untimed, like the reference's load
+    print("[bench] %d windows generated and uploaded in %.1f s" % (n_windows, time.perf_counter() - t_gen),
+          file=sys.stderr, flush=True)
 
     if args.full:
         # the reference's timed region: bootstrap + every transition (main.h:187-293)
@@ -134,7 +154,11 @@ def main():
         wall = time.perf_counter() - t0
         tm0 = dict(kernel_ms=0.0, launches=0)
     else:
+        # every chain starts at its window's teacher weights (the region the burn-in of the whole job ends
+        # in) with the adapted step size, so that the timed transitions accept at the rate the job's do
         s.init_chains(None)
+        for c in range(n_chains):
+            s.set_chain_state(c, teachers[c // cpw], args.eps0, 0, 0)
         steps, warm = args.steps, args.warmup
         if warm:
             s.run(warm)
@@ -143,18 +167,24 @@ def main():
         s.run(steps)  # synchronous at return: the stream is drained
         wall = time.perf_counter() - t0
     tm1 = s.timing()
-    st = s.get_chain_state(0)
+    states = [s.get_chain_state(c) for c in range(n_chains)]
+    stored = s.get_samples(0).shape[0]
     s.close()
+    n_acc = sum(st["n_accepted"] for st in states)
+    n_done = sum(st["transitions_done"] for st in states)
 
     evals = n_chains * steps * args.leapfrog + (n_chains if args.full else 0)
     value = evals / wall
+    ms_per_step = wall * 1e3 / steps
     # dominant kernel: the trajectory kernel.  Average launch duration from HIP events recorded on the
     # sampler's stream around the launches of the timed region.
     dev_ms = tm1["kernel_ms"] - tm0["kernel_ms"]
     launches = tm1["launches"] - tm0["launches"]
     ms_per_launch = dev_ms / max(1, launches)
-    flop_per_launch = flop_per_eval * (n_chains * steps * args.leapfrog) / max(1, launches)
-    achieved = flop_per_launch / (ms_per_launch * 1e-3) / 1e12
+    evals_per_launch = (n_chains * steps * args.leapfrog) / max(1, launches)
+    achieved = flop_per_eval * evals_per_launch / (ms_per_launch * 1e-3) / 1e12
+    kernel_key = "hmc_kernel_wide_64x128" if wide else "hmc_kernel_%s_22x40" % args.layer
+    bytes_per_eval = measured_traffic(kernel_key)
 
     out = {
         "metric": "leapfrog grad-evals/sec (minutes for 200 windows x 800 samples derived), 1 MI355X",
@@ -163,38 +193,47 @@ def main():
         "n_gpus": 1,
         "steps": steps,
         "warmup": warm,
-        "ms_per_step": wall * 1e3 / steps,
+        "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "configs[%d]: %d independent windows x %d chain(s) (%d chains resident per launch), "
-                        "%d->%d->1 BNN, %dx%d features ~N(0,1), teacher-MLP targets + N(0,0.01^2), Gaussian "
-                        "likelihood and prior, %d leapfrog steps per transition" % (
+            "workload": "configs[%d]: %d independent windows x %d chain(s), all resident in HBM (%d chains in "
+                        "flight per launch), %d->%d->1 BNN, %dx%d features ~N(0,1), teacher-MLP targets + "
+                        "N(0,0.01^2), Gaussian likelihood and prior, %d leapfrog steps per transition; one step "
+                        "= one transition of every window, samples stored in the timed region" % (
                             4 if wide else 2, n_windows, cpw, min(n_chains, resident), d0, d1, n_rows, d0,
                             args.leapfrog),
             "layer": args.layer, "cus_per_chain": group, "wgs_per_cu": wgs_per_cu,
-            "workgroups": tm1["workgroups"], "compute_units": cus,
+            "workgroups_last_launch": tm1["workgroups"], "compute_units": cus,
             "transitions_per_launch": args.transitions_per_launch,
-            "eps0": float(hmc.eps0),
+            "eps0": float(hmc.eps0), "adapt_steps": int(hmc.adapt_steps),
+            "samples_stored_per_chain": int(stored),
         },
-        "minutes_200x800": None if wide else EVALS_200x800 / value / 60.0,
-        "minutes_200x800_kind": "not defined for this shape" if wide else (
-            "measured: the whole job was run" if args.full else "extrapolated from the timed transitions"),
-        "minutes_200x1600_extrapolated": None if wide else EVALS_200x1600 / value / 60.0,
+        # 100 burn-in + 800 kept transitions of all 200 windows, plus the bootstrap evaluation (one
+        # gradient evaluation per window: 1/1000 of a step)
+        "minutes_200x800": None if wide or n_windows != 200 else (
+            wall / 60.0 if args.full else (900 + 0.001) * ms_per_step / 6e4),
+        "minutes_200x800_kind": "not defined for this workload" if wide or n_windows != 200 else (
+            "measured: the whole job was run" if args.full else
+            "900 x the measured time of one transition of all 200 windows"),
+        "minutes_200x1600": None if wide or n_windows != 200 else (1700 + 0.001) * ms_per_step / 6e4,
         "reference_minutes_200x800_1xA100_tf32": 42,
-        "accept_rate_chain0": st["n_accepted"] / max(1, st["transitions_done"]),
-        "eps_chain0": st["eps"],
+        "accept_rate": n_acc / max(1, n_done),
+        "eps_chain0": states[0]["eps"],
         "roofline": {
             "bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": achieved / PEAK_TFLOPS,
-            "traffic": (TRAFFIC_BYTES_PER_EVAL_MFMA * n_windows * steps * args.leapfrog / max(1, launches)
-                        if args.layer == "mfma" and not wide else None),
-            "traffic_unit": "bytes per launch (measured offline with rocprofv3 --pmc, see profiles/)",
+            "traffic": None if bytes_per_eval is None else bytes_per_eval * evals_per_launch,
+            "traffic_unit": "HBM bytes per launch: rocprofv3 FETCH_SIZE + WRITE_SIZE per gradient evaluation "
+                            "(profiles/traffic.json) x the evaluations of an average launch",
+            # compulsory bytes: a chain's rows (X and y) once per trajectory
+            "algorithmic_bytes_per_launch": (n_rows * (d0 + 1) * 4) * evals_per_launch / args.leapfrog,
             "kernel": "hmc_kernel_wide" if wide else "hmc_kernel", "launches": launches,
             "ms_per_launch": ms_per_launch, "flop_per_grad_eval": flop_per_eval,
+            "grad_evals_per_launch": evals_per_launch,
         },
     }
     if args.cpu_seconds > 0:
