@@ -121,11 +121,26 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
                      float* grad_cur, float* grad_next, float* loss_values, void* workspace,
                      size_t workspace_bytes, float eps, int lp_steps, void* stream);
 
+/* bnnhmc_mcmc_step for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the same operator with the same arguments
+ * but no workspace -- the exchange scratch is a static device array inside the library (4.5 MiB on
+ * every GPU the library runs on, held until the process ends), and the call allocates nothing.  It
+ * has no counterpart in the reference.  Configurations whose scratch would not fit (see
+ * bnnhmc_step_workspace_bytes) are refused with BNNHMC_ERR_INVALID.  All calls on one GPU share the
+ * array: calls that overlap on one GPU (two streams, two threads) race; calls issued one after the
+ * other on one stream do not.  Check the outcome with bnnhmc_step_check(model, launch, NULL, stream). */
+int bnnhmc_mcmc_step_static(const bnnhmc_model* model, const bnnhmc_launch* launch, const float* x,
+                            const float* y, const float* weights_prev, float* weights_next,
+                            const float* mom_prev, float* mom_next, const float* grad_prev,
+                            float* grad_cur, float* grad_next, float* loss_values, float eps,
+                            int lp_steps, void* stream);
+
 /* Synchronises `stream` and reports whether the last bnnhmc_mcmc_step on this workspace ran to
  * completion: BNNHMC_ERR_TIMEOUT if a bounded in-kernel wait expired (the outputs were then not
  * written), BNNHMC_ERR_DIVERGED if the workgroups did not all hold the same state at the end.  Every
  * bnnhmc_mcmc_step clears the record of the one before it, so check each step whose outcome matters.
- * `launch` is not needed (the record sits at the start of the workspace) and may be NULL.  Stands in
+ * `launch` is not needed (the record sits at the start of the workspace) and may be NULL; workspace
+ * NULL means the library's own scratch (bnnhmc_mcmc_step_static) on the current GPU.  Stands in
  * for the CUDA_CHECK after the launch (include/mcmc/mcmc_step_ffma.h:412). */
 int bnnhmc_step_check(const bnnhmc_model* model, const bnnhmc_launch* launch, void* workspace,
                       void* stream);

@@ -49,7 +49,7 @@ class BnnHmcError(RuntimeError):
 EXPORTS = [
     "bnnhmc_default_model", "bnnhmc_default_hmc", "bnnhmc_default_launch", "bnnhmc_num_params",
     "bnnhmc_last_error", "bnnhmc_device_info", "bnnhmc_step_workspace_bytes", "bnnhmc_mcmc_step",
-    "bnnhmc_step_check", "bnnhmc_sample_momentum", "bnnhmc_log_acpt", "bnnhmc_get_loss_values",
+    "bnnhmc_mcmc_step_static", "bnnhmc_step_check", "bnnhmc_sample_momentum", "bnnhmc_log_acpt", "bnnhmc_get_loss_values",
     "bnnhmc_create", "bnnhmc_destroy", "bnnhmc_set_window_data", "bnnhmc_generate_window",
     "bnnhmc_generate_window_host", "bnnhmc_rng_word", "bnnhmc_rng_normal", "bnnhmc_rng_log_uniform",
     "bnnhmc_get_window_data", "bnnhmc_init_chains", "bnnhmc_run", "bnnhmc_get_samples",
@@ -177,6 +177,13 @@ class Lib:
             C.byref(model), C.byref(launch), _vp(x), _vp(y), _vp(w_prev), _vp(w_next), _vp(m_prev),
             _vp(m_next), _vp(g_prev), _vp(g_cur), _vp(g_next), _vp(loss), _vp(workspace),
             C.c_size_t(workspace_bytes), C.c_float(eps), C.c_int(lp_steps), _vp(stream)))
+
+    def mcmc_step_static(self, model, launch, x, y, w_prev, w_next, m_prev, m_next, g_prev, g_cur, g_next,
+                         loss, eps, lp_steps, stream=0):
+        self.check(self.c.bnnhmc_mcmc_step_static(
+            C.byref(model), C.byref(launch), _vp(x), _vp(y), _vp(w_prev), _vp(w_next), _vp(m_prev),
+            _vp(m_next), _vp(g_prev), _vp(g_cur), _vp(g_next), _vp(loss), C.c_float(eps),
+            C.c_int(lp_steps), _vp(stream)))
 
     def step_check(self, model, launch, workspace, stream=0):
         self.check(self.c.bnnhmc_step_check(C.byref(model), C.byref(launch), _vp(workspace), _vp(stream)))

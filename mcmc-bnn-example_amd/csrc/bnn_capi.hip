@@ -387,7 +387,33 @@ constexpr int LOSS_SLOTS = 64;
 constexpr int MAX_DEVICES = 16;
 static __device__ __align__(256) float g_loss_slots[LOSS_SLOTS][2];
 
+// Exchange scratch of bnnhmc_mcmc_step_static: partial-gradient records, barrier and status words of
+// one step operator call at a time per GPU.  4.5 MiB covers the largest configurations built (one
+// chain on 256 workgroups for 22 -> 40 -> 1, on 64 for 64 -> 128 -> 1).  Every GPU the library runs on
+// holds its own copy until the process ends; host code reaches it only through the address looked up
+// once per device below (the array's name is a host-side stand-in, not a device address).
+constexpr size_t STEP_SCRATCH_BYTES = 4608u * 1024u;
+static __device__ __align__(256) unsigned char g_step_scratch[STEP_SCRATCH_BYTES];
+
 namespace {
+void* g_step_scratch_ptr[MAX_DEVICES] = {nullptr};
+
+int step_scratch(void** out) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= MAX_DEVICES)
+    return fail(BNNHMC_ERR_INVALID, "device index %d is beyond the %d this library keeps state for", dev,
+                MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  if (!g_step_scratch_ptr[dev]) {
+    void* p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_step_scratch)));
+    g_step_scratch_ptr[dev] = p;
+  }
+  *out = g_step_scratch_ptr[dev];
+  return BNNHMC_OK;
+}
+
 float* g_loss_slots_ptr[MAX_DEVICES] = {nullptr};
 unsigned g_loss_next = 0;
 
@@ -673,16 +699,20 @@ static int step_group(const bnnhmc_launch* launch, int resident_wgs, int cap) {
 
 size_t bnnhmc_step_workspace_bytes(const bnnhmc_model* model, const bnnhmc_launch* launch) {
   if (!model) return 0;
-  // sized for the default group (256) when none is configured, whatever device is present
-  const int G = launch && launch->cus_per_chain > 0 ? launch->cus_per_chain : 256;
+  // sized for the largest default group when none is configured (256 workgroups; 64 for the
+  // 64 -> 128 -> 1 kernel), whatever device is present
+  const int G = launch && launch->cus_per_chain > 0 ? launch->cus_per_chain
+                                                    : (model->d0 == 64 && model->d1 == 128 ? 64 : 256);
   return workspace_bytes_for(make_layout(model->d0, model->d1).P, G, 1);
 }
 
-int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, const float* x,
-                     const float* y, const float* weights_prev, float* weights_next,
-                     const float* mom_prev, float* mom_next, const float* grad_prev,
-                     float* grad_cur, float* grad_next, float* loss_values, void* workspace,
-                     size_t workspace_bytes, float eps, int lp_steps, void* stream) {
+// The step operator on a given exchange scratch; allocates nothing (device and plan queries happen on
+// the first call for a configuration only, and allocate nothing either).
+static int mcmc_step_on(const bnnhmc_model* model, const bnnhmc_launch* launch, const float* x,
+                        const float* y, const float* weights_prev, float* weights_next,
+                        const float* mom_prev, float* mom_next, const float* grad_prev,
+                        float* grad_cur, float* grad_next, float* loss_values, void* workspace,
+                        size_t workspace_bytes, float eps, int lp_steps, void* stream) {
   int rc = check_model(model);
   if (rc) return rc;
   if (!x || !y || !weights_prev || !weights_next || !mom_prev || !mom_next || !grad_prev ||
@@ -752,10 +782,42 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
   return BNNHMC_OK;
 }
 
+int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, const float* x,
+                     const float* y, const float* weights_prev, float* weights_next,
+                     const float* mom_prev, float* mom_next, const float* grad_prev,
+                     float* grad_cur, float* grad_next, float* loss_values, void* workspace,
+                     size_t workspace_bytes, float eps, int lp_steps, void* stream) {
+  return mcmc_step_on(model, launch, x, y, weights_prev, weights_next, mom_prev, mom_next, grad_prev,
+                      grad_cur, grad_next, loss_values, workspace, workspace_bytes, eps, lp_steps, stream);
+}
+
+int bnnhmc_mcmc_step_static(const bnnhmc_model* model, const bnnhmc_launch* launch, const float* x,
+                            const float* y, const float* weights_prev, float* weights_next,
+                            const float* mom_prev, float* mom_next, const float* grad_prev,
+                            float* grad_cur, float* grad_next, float* loss_values, float eps,
+                            int lp_steps, void* stream) {
+  if (!model) return fail(BNNHMC_ERR_INVALID, "model is null");
+  const size_t need = bnnhmc_step_workspace_bytes(model, launch);
+  if (need > STEP_SCRATCH_BYTES)
+    return fail(BNNHMC_ERR_INVALID,
+                "this configuration needs %zu bytes of exchange scratch; bnnhmc_mcmc_step_static holds %zu "
+                "(use bnnhmc_mcmc_step with a workspace of your own)",
+                need, (size_t)STEP_SCRATCH_BYTES);
+  void* scratch = nullptr;
+  const int rc = step_scratch(&scratch);
+  if (rc) return rc;
+  return mcmc_step_on(model, launch, x, y, weights_prev, weights_next, mom_prev, mom_next, grad_prev,
+                      grad_cur, grad_next, loss_values, scratch, STEP_SCRATCH_BYTES, eps, lp_steps, stream);
+}
+
 int bnnhmc_step_check(const bnnhmc_model* model, const bnnhmc_launch* launch, void* workspace,
                       void* stream) {
   (void)launch;
-  if (!model || !workspace) return fail(BNNHMC_ERR_INVALID, "null argument to bnnhmc_step_check");
+  if (!model) return fail(BNNHMC_ERR_INVALID, "null argument to bnnhmc_step_check");
+  if (!workspace) {  // the step ran on the library's own scratch (bnnhmc_mcmc_step_static)
+    const int rc = step_scratch(&workspace);
+    if (rc) return rc;
+  }
   // the status words sit at the start of the workspace whatever the launch parameters were
   return read_status(workspace, (hipStream_t)stream);
 }
