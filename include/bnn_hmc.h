@@ -73,8 +73,7 @@ typedef struct bnnhmc_launch {
   int layer;          /* BNNHMC_LAYER_MFMA (v_mfma_f32_16x16x4_f32) or BNNHMC_LAYER_FFMA          */
   int cus_per_chain;  /* workgroups that share one chain's rows; 0 = default: 4 for a sampler (64   */
                       /* chains in flight on 256 CUs; a smaller last batch is widened to fill the   */
-                      /* device, up to 256 per chain), 256 for the step operator; the              */
-                      /* 64 -> 128 -> 1 network takes at most 64                                    */
+                      /* device, up to 256 per chain), 256 for the step operator                    */
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */
   int threads;        /* threads per workgroup; default 512 for MFMA (every tile loop), 256 for  */
                       /* FFMA and with wgs_per_cu = 2.  The plain MFMA loop is also built for    */

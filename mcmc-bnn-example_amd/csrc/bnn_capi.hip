@@ -165,8 +165,8 @@ int make_plan_uncached(const bnnhmc_model& m, const bnnhmc_launch* lp, const Dev
   if (p.wide) {
     if (l.layer != BNNHMC_LAYER_MFMA)
       return fail(BNNHMC_ERR_INVALID, "64 -> 128 -> 1 is built for the MFMA layer only");
-    if (l.cus_per_chain > 64)
-      return fail(BNNHMC_ERR_INVALID, "64 -> 128 -> 1 supports at most 64 workgroups per chain, got %d",
+    if (l.cus_per_chain > 256)
+      return fail(BNNHMC_ERR_INVALID, "64 -> 128 -> 1 supports at most 256 workgroups per chain, got %d",
                   l.cus_per_chain);
     p.threads = l.threads > 0 ? l.threads : 256;
     p.kernel = hmc_kernel_wide_for(m.d0, m.d1, m.lik_kind, p.threads, &p.dyn_lds, &p.wg_scratch_floats);
@@ -388,8 +388,9 @@ constexpr int MAX_DEVICES = 16;
 static __device__ __align__(256) float g_loss_slots[LOSS_SLOTS][2];
 
 // Exchange scratch of bnnhmc_mcmc_step_static: partial-gradient records, barrier and status words of
-// one step operator call at a time per GPU.  4.5 MiB covers the largest configurations built (one
-// chain on 256 workgroups for 22 -> 40 -> 1, on 64 for 64 -> 128 -> 1).  Every GPU the library runs on
+// one step operator call at a time per GPU.  4.5 MiB covers one chain on 256 workgroups for
+// 22 -> 40 -> 1 and on up to 64 workgroups for 64 -> 128 -> 1 (wider groups of that network need more and
+// are refused).  Every GPU the library runs on
 // holds its own copy until the process ends; host code reaches it only through the address looked up
 // once per device below (the array's name is a host-side stand-in, not a device address).
 constexpr size_t STEP_SCRATCH_BYTES = 4608u * 1024u;
@@ -525,7 +526,7 @@ KArgs base_args(const bnnhmc_sampler* s) {
 
 int launch_and_count(bnnhmc_sampler* s, KArgs& a, int groups) {
   int wgs = 0;
-  set_grid(a, groups, s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs, s->plan.wide ? 64 : 256) : s->plan.G,
+  set_grid(a, groups, s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs, 256) : s->plan.G,
            &wgs);
   HIP_TRY(launch_fill_u32(a.barrier, (size_t)groups * BARRIER_STRIDE_WORDS, 0u, s->stream));
   HIP_TRY(launch_hmc_kernel(s->plan.kernel, a, wgs, s->plan.threads, s->plan.dyn_lds, s->stream));
@@ -689,7 +690,7 @@ float bnnhmc_rng_log_uniform(uint32_t seed, uint32_t chain_id, uint32_t t) {
 // operator level
 // =================================================================================================
 // workgroups the step operator gives its single chain: the configured count, or by default the
-// largest power of two that is resident at once (at most 256; 64 for the 64 -> 128 -> 1 kernel)
+// largest power of two that is resident at once (at most 256)
 static int step_group(const bnnhmc_launch* launch, int resident_wgs, int cap) {
   if (launch && launch->cus_per_chain > 0) return launch->cus_per_chain;
   int G = 1;
@@ -699,10 +700,8 @@ static int step_group(const bnnhmc_launch* launch, int resident_wgs, int cap) {
 
 size_t bnnhmc_step_workspace_bytes(const bnnhmc_model* model, const bnnhmc_launch* launch) {
   if (!model) return 0;
-  // sized for the largest default group when none is configured (256 workgroups; 64 for the
-  // 64 -> 128 -> 1 kernel), whatever device is present
-  const int G = launch && launch->cus_per_chain > 0 ? launch->cus_per_chain
-                                                    : (model->d0 == 64 && model->d1 == 128 ? 64 : 256);
+  // sized for the default group (256) when none is configured, whatever device is present
+  const int G = launch && launch->cus_per_chain > 0 ? launch->cus_per_chain : 256;
   return workspace_bytes_for(make_layout(model->d0, model->d1).P, G, 1);
 }
 
@@ -728,12 +727,10 @@ static int mcmc_step_on(const bnnhmc_model* model, const bnnhmc_launch* launch, 
   rc = make_plan(*model, launch, di, plan);
   if (rc) return rc;
   const Layout L = make_layout(model->d0, model->d1);
-  const int G = step_group(launch, plan.resident_wgs, plan.wide ? 64 : 256);
+  const int G = step_group(launch, plan.resident_wgs, 256);
   if (G > plan.resident_wgs)
     return fail(BNNHMC_ERR_RESIDENCY, "%d workgroups per chain requested but only %d can be resident", G,
                 plan.resident_wgs);
-  if (plan.wide && G > 64)
-    return fail(BNNHMC_ERR_INVALID, "64 -> 128 -> 1 supports at most 64 workgroups per chain, got %d", G);
   if (workspace_bytes < workspace_bytes_for(L.P, G, 1))
     return fail(BNNHMC_ERR_INVALID, "workspace too small: %zu < %zu bytes", workspace_bytes,
                 workspace_bytes_for(L.P, G, 1));

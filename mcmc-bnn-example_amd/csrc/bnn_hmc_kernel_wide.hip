@@ -431,39 +431,113 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
       ok = group_barrier(counter, a.G, rank, ++bar_epoch, a.status, a.spin_limit, &s_flag,
                          rank != a.debug_drop_rank);
       if (!ok) break;
-      // ---- stage 2: every workgroup adds the G records in rank order, seeded with the prior
-      //      gradient (mcmc_step_ffma.h:144) ----
       const float* grp_part = part_base + (size_t)buf * a.G * SLOT;
-      // a thread takes 16-byte columns of the records, eight loads in flight, records in rank order
-      for (int col = tid; col < P_AL / 4; col += T) {
-        f4 v = {0.f, 0.f, 0.f, 0.f};
-        const float* src = grp_part + 4 * col;
-        for (int r0 = 0; r0 < a.G; r0 += 8) {
-          f4 t8[8];
-          const float* p8[8];
+      if (!a.two_phase) {
+        // ---- stage 2 (up to 64 workgroups per chain): every workgroup adds the G records in rank
+        //      order, seeded with the prior gradient (mcmc_step_ffma.h:144).  A thread takes 16-byte
+        //      columns of the records, eight loads in flight ----
+        for (int col = tid; col < P_AL / 4; col += T) {
+          f4 v = {0.f, 0.f, 0.f, 0.f};
+          const float* src = grp_part + 4 * col;
+          for (int r0 = 0; r0 < a.G; r0 += 8) {
+            f4 t8[8];
+            const float* p8[8];
 #pragma unroll
-          for (int k = 0; k < 8; ++k) p8[k] = src + (size_t)min(r0 + k, a.G - 1) * SLOT;
-          ld_agent4x8(t8, p8);
+            for (int k = 0; k < 8; ++k) p8[k] = src + (size_t)min(r0 + k, a.G - 1) * SLOT;
+            ld_agent4x8(t8, p8);
 #pragma unroll
-          for (int k = 0; k < 8; ++k)
-            if (r0 + k < a.G) v += t8[k];
-        }
+            for (int k = 0; k < 8; ++k)
+              if (r0 + k < a.G) v += t8[k];
+          }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int p = 4 * col + e;
-          if (p < P) s_g[p] = prior_grad(mc, s_w[p]) + v[e];
+          for (int e = 0; e < 4; ++e) {
+            const int p = 4 * col + e;
+            if (p < P) s_g[p] = prior_grad(mc, s_w[p]) + v[e];
+          }
         }
-      }
-      __syncthreads();  // the columns are not the parameters a thread owns in the update loops
-      if (last) {
-        double d = 0.0;
-        for (int r = 0; r < a.G; ++r) {
-          const float lo = ld_agent(grp_part + (size_t)r * SLOT + P_AL);
-          const float hi = ld_agent(grp_part + (size_t)r * SLOT + P_AL + 1);
-          d += bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
-                              __builtin_bit_cast(uint32_t, lo));
+        __syncthreads();  // the columns are not the parameters a thread owns in the update loops
+        if (last) {
+          double d = 0.0;
+          for (int r = 0; r < a.G; ++r) {
+            const float lo = ld_agent(grp_part + (size_t)r * SLOT + P_AL);
+            const float hi = ld_agent(grp_part + (size_t)r * SLOT + P_AL + 1);
+            d += bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
+                                __builtin_bit_cast(uint32_t, lo));
+          }
+          dl_total = d;
         }
-        dl_total = d;
+      } else {
+        // ---- stage 2 (more than 64 workgroups per chain), in two phases: reading all G records in
+        //      every workgroup would move G * G * 34 KB per step.  Phase 1: workgroup `rank` reduces
+        //      the 32-parameter slices rank, rank + G, ... -- one 128-byte line of every record each --
+        //      over all G records: thread (record lane rl = tid / 8, 16-byte column c = tid % 8) adds
+        //      records rl, rl + T/8, ... in order, the record lanes of a wave are added by a fixed xor
+        //      tree and the waves in order through LDS.  Phase 2, once every slice is stored: everyone
+        //      reads the totals. ----
+        float* tot = a.totals + (size_t)group * SLOT;
+        constexpr int RL = T / 8;                  // record lanes of a workgroup
+        constexpr int N_SLICE = (P + 31) / 32;
+        float* s_x = s_red;                        // free: this step's record has been published
+        for (int sl = rank; sl < N_SLICE; sl += a.G) {
+          const int c = tid & 7, rl = tid >> 3;
+          const float* src = grp_part + 32 * sl + 4 * c;
+          f4 v = {0.f, 0.f, 0.f, 0.f};
+          for (int r0 = rl; r0 < a.G; r0 += 8 * RL) {
+            f4 t8[8];
+            const float* p8[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) p8[k] = src + (size_t)min(r0 + RL * k, a.G - 1) * SLOT;
+            ld_agent4x8(t8, p8);
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+              if (r0 + RL * k < a.G) v += t8[k];
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float x = v[e];
+            x += __shfl_xor(x, 8);
+            x += __shfl_xor(x, 16);
+            x += __shfl_xor(x, 32);
+            v[e] = x;
+          }
+          __syncthreads();  // the previous slice's sums have been read
+          if ((tid & 63) < 8) *reinterpret_cast<f4*>(&s_x[32 * wave + 4 * c]) = v;
+          __syncthreads();
+          if (tid < 32 && 32 * sl + tid < P) {
+            float x = s_x[tid];
+#pragma unroll
+            for (int wv = 1; wv < W; ++wv) x += s_x[32 * wv + tid];
+            st_agent(tot + 32 * sl + tid, x);
+          }
+        }
+        if (last && rank == a.G - 1 && wave == W - 1) {
+          const int lane = tid & 63;
+          double d = 0.0;
+          for (int r = lane; r < a.G; r += 64) {
+            const float lo = ld_agent(grp_part + (size_t)r * SLOT + P_AL);
+            const float hi = ld_agent(grp_part + (size_t)r * SLOT + P_AL + 1);
+            d += bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
+                                __builtin_bit_cast(uint32_t, lo));
+          }
+#pragma unroll
+          for (int msk = 1; msk < 64; msk <<= 1) d += shfl_xor_d(d, msk);
+          if (lane == 0) {
+            const uint64_t bits = double_to_bits(d);
+            st_agent(tot + P_AL, __builtin_bit_cast(float, (uint32_t)bits));
+            st_agent(tot + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)));
+          }
+        }
+        // every workgroup has slices to announce (G <= number of slices), everybody waits for all
+        ok = reducer_barrier(counter, a.G, true, rank, bar_epoch, a.status, a.spin_limit, &s_flag,
+                             rank != a.debug_drop_rank);
+        if (!ok) break;
+        for (int p = tid; p < P; p += T) s_g[p] = prior_grad(mc, s_w[p]) + ld_agent(tot + p);
+        if (last) {
+          const float lo = ld_agent(tot + P_AL);
+          const float hi = ld_agent(tot + P_AL + 1);
+          dl_total = bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
+                                    __builtin_bit_cast(uint32_t, lo));
+        }
       }
       buf ^= 1;
     }

@@ -6,6 +6,11 @@
 //                [--lik student_t|gaussian] [--layer mfma|ffma] [--cus-per-chain G] [--wgs-per-cu K]
 //                [--seed S] [--data FILE] [--dump FILE] [--features D0 --hidden D1]   (22 40 or 64 128)
 //
+// --dump FILE writes the kept samples of every chain as a NumPy array file (format 1.0, little-endian
+// float32, shape (chains, samples, parameters), chain = window * chains_per_window + chain of the
+// window) and FILE.json beside it with what a reader needs to interpret it: shapes, layer sizes,
+// model and sampler constants, seed, and per chain the final step size and the accepted transitions.
+//
 // Without --data every window is filled with the synthetic recipe (features ~ N(0,1), targets from
 // a random teacher MLP plus noise).  With --data the reference's text format is read
 // (include/mcmc/io.h:43-86) into window 0 and the features are scaled by 0.001 (main.h:162-164).
@@ -75,6 +80,23 @@ void print_stats(const char* name, const float* d, size_t rows, size_t cols) {
     if (d[i] < mn) mn = d[i];
   }
   std::printf("%s: Shape: %zu x %zu, word: 4, min: %g, max: %g, mean: %g\n", name, rows, cols, mn, mx, mean);
+}
+
+// header of a NumPy array file, format 1.0: magic, version, little-endian header length, a Python
+// dict literal padded with spaces so that the data starts at a multiple of 64 bytes
+void write_npy_header(FILE* f, int chains, int samples, int params) {
+  char dict[192];
+  const int len = std::snprintf(dict, sizeof(dict), "{'descr': '<f4', 'fortran_order': False, 'shape': (%d, %d, %d), }",
+                                chains, samples, params);
+  const int unpadded = 10 + len + 1;  // magic 6 + version 2 + length 2 + dict + newline
+  const int pad = (64 - unpadded % 64) % 64;
+  const unsigned short hlen = (unsigned short)(len + pad + 1);
+  const unsigned char pre[10] = {0x93, 'N', 'U', 'M', 'P', 'Y', 1, 0, (unsigned char)(hlen & 0xff),
+                                 (unsigned char)(hlen >> 8)};
+  std::fwrite(pre, 1, sizeof(pre), f);
+  std::fwrite(dict, 1, (size_t)len, f);
+  for (int i = 0; i < pad; ++i) std::fputc(' ', f);
+  std::fputc('\n', f);
 }
 
 }  // namespace
@@ -149,8 +171,19 @@ int main(int argc, char** argv) {
 
   // ------------------------------------------------------------------ dump (main.h:295-307)
   std::vector<float> samples((size_t)hmc.n_samples * P);
-  FILE* out = o.dump.empty() ? nullptr : std::fopen(o.dump.c_str(), "wb");
-  for (int c = 0; c < o.windows * o.chains; ++c) {
+  const int n_chains = o.windows * o.chains;
+  int stored_all = 0;
+  CHECK(bnnhmc_get_samples(s, 0, nullptr, &stored_all));
+  FILE* out = nullptr;
+  if (!o.dump.empty()) {
+    out = std::fopen(o.dump.c_str(), "wb");
+    if (!out) {
+      std::fprintf(stderr, "error: cannot open %s for writing\n", o.dump.c_str());
+      return 1;
+    }
+    write_npy_header(out, n_chains, stored_all, P);
+  }
+  for (int c = 0; c < n_chains; ++c) {
     int stored = 0;
     CHECK(bnnhmc_get_samples(s, c, samples.data(), &stored));
     if (c == 0) print_stats("Final samples", samples.data(), stored, P);
@@ -158,8 +191,39 @@ int main(int argc, char** argv) {
   }
   if (out) {
     std::fclose(out);
-    std::printf("Wrote %d chain(s) x %d samples x %d floats to %s\n", o.windows * o.chains,
-                hmc.n_samples, P, o.dump.c_str());
+    const std::string meta = o.dump + ".json";
+    FILE* mj = std::fopen(meta.c_str(), "w");
+    if (!mj) {
+      std::fprintf(stderr, "error: cannot open %s for writing\n", meta.c_str());
+      return 1;
+    }
+    std::fprintf(mj,
+                 "{\n \"format\": \"npy float32 little-endian, C order\",\n \"shape\": [%d, %d, %d],\n"
+                 " \"axes\": [\"chain = window * chains_per_window + chain of the window\", \"kept sample\", "
+                 "\"parameter: W1[k * hidden + c] | b1[c] | w2[c] | b2\"],\n"
+                 " \"windows\": %d,\n \"chains_per_window\": %d,\n \"features\": %d,\n \"hidden\": %d,\n"
+                 " \"rows\": %d,\n \"parameters\": %d,\n \"likelihood\": \"%s\",\n \"lik_scale\": %.17g,\n"
+                 " \"lik_df\": %.17g,\n \"prior_scale\": %.17g,\n \"leapfrog_steps\": %d,\n \"burn_in\": %d,\n"
+                 " \"adapt_steps\": %d,\n \"eps0\": %.9g,\n \"seed\": %u,\n \"data\": \"%s\",\n \"chains\": [",
+                 n_chains, stored_all, P, o.windows, o.chains, model.d0, model.d1, model.n, P,
+                 model.lik_kind == BNNHMC_LIK_GAUSSIAN ? "gaussian" : "student_t", model.lik_scale,
+                 model.lik_kind == BNNHMC_LIK_GAUSSIAN ? 0.0 : model.lik_df, model.prior_scale,
+                 hmc.leapfrog_steps, hmc.burn_in, hmc.adapt_steps, (double)hmc.eps0, hmc.seed,
+                 o.data.empty() ? "synthetic: features ~ N(0,1), teacher MLP ~ N(0, 0.1^2), noise sigma 0.01, "
+                                  "key (seed, window)"
+                                : o.data.c_str());
+    for (int c = 0; c < n_chains; ++c) {
+      float ceps = 0;
+      int cacc = 0, cdone = 0;
+      CHECK(bnnhmc_get_chain_state(s, c, nullptr, nullptr, &ceps, &cdone, &cacc));
+      std::fprintf(mj, "%s\n  {\"chain\": %d, \"window\": %d, \"final_eps\": %.9g, \"transitions\": %d, "
+                       "\"accepted\": %d}",
+                   c ? "," : "", c, c / o.chains, (double)ceps, cdone, cacc);
+    }
+    std::fprintf(mj, "\n ]\n}\n");
+    std::fclose(mj);
+    std::printf("Wrote %d chain(s) x %d samples x %d floats to %s (metadata in %s)\n", n_chains, stored_all,
+                P, o.dump.c_str(), meta.c_str());
   }
   double l1 = 0, l2 = 0, fl = 0;
   if (hmc.n_samples > 0) {

@@ -495,11 +495,36 @@ def test_host_driver_runs_init_run_dump(pkg, tmp_path):
 
     exe = os.path.join(pkg.PKG_DIR, "bnn_hmc_main")
     assert os.path.exists(exe), "driver not built"
-    dump = tmp_path / "chain.bin"
-    r = subprocess.run([exe, "--windows", "2", "--rows", "2048", "--samples", "6", "--burn-in", "4",
-                        "--leapfrog", "20", "--dump", str(dump)], capture_output=True, text=True, timeout=120)
+    dump = tmp_path / "chain.npy"
+    r = subprocess.run([exe, "--windows", "2", "--chains", "2", "--rows", "2048", "--samples", "6", "--burn-in",
+                        "4", "--leapfrog", "20", "--seed", "5", "--dump", str(dump)], capture_output=True,
+                       text=True, timeout=120)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "Final samples: Shape: 6 x 961" in r.stdout and "Final loss1:" in r.stdout
     assert "MCMC (4 burn in, 6 sample steps, 20 leap-frog steps) done in" in r.stdout
-    data = np.fromfile(dump, np.float32)
-    assert data.size == 2 * 6 * 961 and np.all(np.isfinite(data))
+    # the dump is a NumPy array file plus a JSON sidecar that lets a reader interpret it
+    import json
+
+    data = np.load(dump, allow_pickle=False)
+    assert data.dtype == np.float32 and data.shape == (4, 6, 961) and np.all(np.isfinite(data))
+    meta = json.load(open(str(dump) + ".json"))
+    assert meta["shape"] == [4, 6, 961] and meta["windows"] == 2 and meta["chains_per_window"] == 2
+    assert (meta["features"], meta["hidden"], meta["rows"], meta["parameters"]) == (22, 40, 2048, 961)
+    assert meta["likelihood"] == "student_t" and meta["lik_scale"] == 100.0 and meta["lik_df"] == 2.2
+    assert meta["prior_scale"] == 200.0 and meta["seed"] == 5 and meta["leapfrog_steps"] == 20
+    assert meta["burn_in"] == 4 and len(meta["chains"]) == 4
+    for c, row in enumerate(meta["chains"]):
+        assert row["chain"] == c and row["window"] == c // 2 and row["transitions"] == 10
+        assert 0 <= row["accepted"] <= 10 and row["final_eps"] > 0
+    # the same chains through the library directly: the file holds exactly their samples
+    lib = pkg.load()
+    s = lib.create(lib.default_model(n=2048), lib.default_hmc(leapfrog_steps=20, burn_in=4, n_samples=6, seed=5),
+                   lib.default_launch(), 2, 2)
+    for w in range(2):
+        s.generate_window(w, teacher_scale=0.1, noise_sigma=0.01)
+    s.init_chains(None)
+    s.run(10)
+    for c in range(4):
+        assert s.get_samples(c).tobytes() == data[c].tobytes()
+        assert s.get_chain_state(c)["n_accepted"] == meta["chains"][c]["accepted"]
+    s.close()

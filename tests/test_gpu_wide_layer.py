@@ -47,14 +47,14 @@ def test_layer_sizes_are_checked(pkg, lib):
     with pytest.raises(pkg.BnnHmcError):  # no FFMA variant of the wide network
         lib.create(lib.default_model(d0=D0, d1=D1, n=16), lib.default_hmc(),
                    lib.default_launch(layer=pkg.LAYER_FFMA), 1, 1)
-    with pytest.raises(pkg.BnnHmcError):  # groups wider than 64 are not built for it
+    with pytest.raises(pkg.BnnHmcError):  # at most 256 workgroups per chain
         lib.create(lib.default_model(d0=D0, d1=D1, n=16), lib.default_hmc(),
-                   lib.default_launch(cus_per_chain=128), 1, 1)
+                   lib.default_launch(cus_per_chain=512), 1, 1)
 
 
 @pytest.mark.parametrize("kind", ["t", "gauss"])
 @pytest.mark.parametrize("n,G", [(1, 1), (3, 2), (16, 1), (17, 4), (100, 3), (1000, 8), (4101, 32),
-                                 (9000, 64), (58368, 0), (233472, 64)])
+                                 (9000, 64), (58368, 0), (233472, 64), (9000, 96), (40000, 128), (233472, 256)])
 def test_eval_matches_oracle(pkg, lib, orc, kind, n, G):
     say("wide eval lik=%s n=%d G=%d" % (kind, n, G))
     model, om, gen = models(pkg, lib, kind, n)
@@ -99,7 +99,8 @@ def test_eval_is_deterministic(pkg, lib, orc):
 @pytest.mark.parametrize("kind,n,L,eps,G,offset", [("t", 777, 1, 0.01, 4, 0), ("t", 2048, 2, 0.01, 8, 0),
                                                    ("t", 1500, 25, 0.003, 32, 0), ("gauss", 999, 10, 1e-5, 5, 0),
                                                    ("gauss", 4096, 40, 1e-5, 64, 0), ("t", 20000, 12, 0.003, 0, 0),
-                                                   ("t", 333, 3, 0.01, 2, 4)])
+                                                   ("t", 333, 3, 0.01, 2, 4), ("t", 30000, 10, 0.003, 128, 0),
+                                                   ("gauss", 58368, 6, 1e-5, 256, 0)])
 def test_mcmc_step_operator_matches_oracle(pkg, lib, orc, kind, n, L, eps, G, offset):
     say("wide mcmc_step lik=%s n=%d L=%d G=%d offset=%d" % (kind, n, L, G, offset))
     model, om, gen = models(pkg, lib, kind, n)
@@ -132,11 +133,14 @@ def test_mcmc_step_operator_matches_oracle(pkg, lib, orc, kind, n, L, eps, G, of
     np.testing.assert_allclose(loss[n:], losso[n:], rtol=1e-6, atol=1e-6)
 
 
-def test_transitions_match_oracle_decisions(pkg, lib, orc):
+@pytest.mark.parametrize("G", [8, 128])
+def test_transitions_match_oracle_decisions(pkg, lib, orc, G):
+    """G = 8: every workgroup adds all records; G = 128: the two-phase exchange (each workgroup reduces
+    slices of the parameters, all read the totals)."""
     n, L, burn, keep, seed = 1024, 12, 20, 20, 33
     model, om, gen = models(pkg, lib, "t_stiff", n)
     hmc = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=0.004, seed=seed)
-    s = lib.create(model, hmc, lib.default_launch(cus_per_chain=8, transitions_per_launch=7), 1, 1)
+    s = lib.create(model, hmc, lib.default_launch(cus_per_chain=G, transitions_per_launch=7), 1, 1)
     s.generate_window(0, **gen)
     X, y = s.get_window_data(0)
     s.init_chains(None)
