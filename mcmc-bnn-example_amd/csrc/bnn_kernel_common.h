@@ -30,6 +30,35 @@ __device__ __forceinline__ float row16_allreduce(float v) {
   v += dpp_move<0x140>(v);  // row_mirror
   return v;
 }
+// Four sums over the 16 lanes of a DPP row at once, in 8 instructions instead of 4 x 4: the four
+// values are first folded into each other across the four banks of four lanes (writes masked by
+// bank), so that bank j of the result holds the sum of v_j -- the same bits in its four lanes (the
+// last two steps add a value to its mirror image).  row16_bcast<j> then hands bank j to all 16 lanes.
+// Written in assembly because a bank-masked DPP add has no builtin; a DPP instruction must not read a
+// register the instruction before it (or the one before that) wrote, hence the s_nops.
+__device__ __forceinline__ float row16_reduce4(float v0, float v1, float v2, float v3) {
+  float r01, r23, z;
+  asm("s_nop 1\n\t"
+      "v_add_f32_dpp %[r01], %[v0], %[v0] row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %[r23], %[v2], %[v2] row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %[r01], %[v1], %[v1] row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+      "v_add_f32_dpp %[r23], %[v3], %[v3] row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+      "s_nop 0\n\t"
+      "v_add_f32_dpp %[z], %[r01], %[r01] row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %[z], %[r23], %[r23] row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "s_nop 1\n\t"
+      "v_add_f32_dpp %[z], %[z], %[z] quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 1\n\t"
+      "v_add_f32_dpp %[z], %[z], %[z] quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf"
+      : [r01] "=&v"(r01), [r23] "=&v"(r23), [z] "=&v"(z)
+      : [v0] "v"(v0), [v1] "v"(v1), [v2] "v"(v2), [v3] "v"(v3));
+  return z;
+}
+template <int J>
+__device__ __forceinline__ float row16_bcast(float z) {
+  return dpp_move<0x150 + 4 * J>(z);  // row_newbcast: lane 4 J of each row to its 16 lanes
+}
+
 // sum over the 8 lanes of a half row
 __device__ __forceinline__ float row8_allreduce(float v) {
   v += dpp_move<0xB1>(v);

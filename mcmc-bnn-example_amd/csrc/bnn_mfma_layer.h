@@ -1,0 +1,575 @@
+// The MFMA layer of the 22 -> 40 -> 1 trajectory kernel: both contractions of a 16-row tile on
+// v_mfma_f32_16x16x4_f32, the pointwise stage between them, and the tile loops.  In a header of its own
+// so that the tile-ceiling probe (tile_ceiling.hip) times exactly the code the kernel runs.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "bnn_device.h"
+#include "bnn_kernel_common.h"
+
+namespace bnn {
+
+// Constant operand slots of the MFMA layer: `one` reads (1, 0) at offsets j * D0 (j < 4), `zero` reads
+// (0, 0); lanes holding the appended constant-one feature or tile padding point here.
+template <int D0>
+struct AugTable {
+  float one[3 * D0 + 4];
+  float zero[3 * D0 + 4];
+};
+template <int D0>
+constexpr AugTable<D0> make_aug_table() {
+  AugTable<D0> t{};
+  for (int j = 0; j < 4; ++j) t.one[j * D0] = 1.0f;
+  return t;
+}
+__device__ const AugTable<22> k_aug_table_22 = make_aug_table<22>();
+template <int D0>
+__device__ __forceinline__ const AugTable<D0>* aug_table();
+template <>
+__device__ __forceinline__ const AugTable<22>* aug_table<22>() {
+  return &k_aug_table_22;
+}
+
+// ================================================================================================
+// MFMA layer: both contractions on v_mfma_f32_16x16x4_f32.
+//
+// Lane l = 16 q + n (q = 0..3, n = 0..15).  A 16-row tile is processed as
+//   GEMM1  A = X_aug tile  [16 rows x K]   lane (n, q) holds row n, k = KS q + s      (s < KS)
+//          B = W1_aug      [K x 16 c]      lane (n, q) holds k = KS q + s, c = 16 t + n
+//          C = pre-act     [16 rows x 16 c] lane (n, q) holds rows 4 q + j, c = 16 t + n
+//   GEMM2  A = delta^T     [16 c x 4 rows]  = C layout of GEMM1 reused as is (k-step j <-> rows
+//                                             4 q + j): no shuffle between the two GEMMs
+//          B = X_aug tile  [4 rows x 16 f]  lane (n, q) holds row 4 q + j, features 2 n + u
+//          C = dW1_aug^T   [16 c x 16 f]    lane (n, q) holds c = 16 t + 4 q + j', f = 2 n + u
+// X_aug appends a constant-one feature (index D0) so that b1 rides in GEMM1 and db1 falls out of
+// GEMM2; the contraction index of GEMM1 and the feature index of GEMM2 are permuted so that every
+// lane reads contiguous floats of a row.
+// ================================================================================================
+template <int D0, int D1, int PIPE>
+struct MfmaLayer {
+  static_assert(D0 % 2 == 0, "feature pairs are read as float2");
+  static constexpr int KS = (D0 + 1 + 3) / 4;  // k-steps of GEMM1 (one more feature: the bias)
+  static_assert(KS % 2 == 0, "k-steps are read in pairs");
+  static constexpr int KP = KS / 2;
+  static constexpr int NT = (D1 + 15) / 16;  // hidden tiles
+  static_assert(D0 + 1 <= 32, "one feature-pair tile");
+  static constexpr int oB1 = D0 * D1, oW2 = oB1 + D1, oB2 = oW2 + D1, P = oB2 + 1;
+  static constexpr int P_AL = (P + 3) / 4 * 4;
+
+  // The activation is carried as the logistic value s = 1 / (1 + 2^t) = (h + 1) / 2 and h = tanh is
+  // never formed: the layer-2 dot, the layer-2 weight gradient and 1 - h^2 = 4 s (1 - s) are all
+  // affine in s or products of s, and the constants move into per-step operands (one VALU
+  // instruction less per hidden value and row).
+  float w1b[KS][NT];   // W1_aug scaled by -2/ln 2: GEMM1 yields the exp2 argument t of the activation
+  float w2g[NT];       // -2 w2[c] k2: the layer-2 dot yields r = (y - yhat - b2) k2, where k2 is the power
+                       // of two next to k = 1/scale^2 (Gaussian: r k / k2 is the per-row loss gradient)
+                       // or k = 1/scale (Student-t: r k / k2 is the scaled residual).  A power of two
+                       // keeps the coefficients exact: the dot cancels from terms of size |w2| k to a
+                       // residual thousands of times smaller, and a rounding error in a coefficient
+                       // would be the same in every row and add up over the rows instead of averaging out
+  float y_k;           // k2 in lane n == 0, else 0
+  float y_0;           // the constant part of the dot, (sum_c w2[c] - b2) k2, computed in double and
+                       // split over lanes n == 0 (leading part) and n == 1 (remainder)
+  float ratio;         // k / k2 (exact)
+  f4 dacc[NT][2];      // sum over rows of s (1 - s) g' x_aug, g' = g k2 / k (Gaussian) or g (Student-t)
+  float dw2s[NT];      // sum over rows of g' s
+                       // (in the lanes of the padded hidden units, where s is exactly 1/2, this is half the
+                       // sum over rows of g', added in the very order of the other lanes' sums: dw2 =
+                       // 2 (dw2s - that) is then exactly zero where every s is 1/2 -- all weights zero,
+                       // the reference's start)
+  double dl;
+
+  struct TileIn {
+    f2 xa[KP];
+    f2 xb[4];
+    f4 yv;
+  };
+
+  static constexpr float kExp2Scale = -2.88539008177792681472f;  // -2 / ln 2, kernel_helpers.h:37
+
+  template <int LIK>
+  __device__ __forceinline__ void load_weights(const float* s_w, const ModelConsts& mc) {
+    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    const float k = LIK == 1 ? mc.scale_recp * mc.scale_recp : mc.scale_recp;
+    // the power of two next to k, and its reciprocal
+    const uint32_t k2_bits = (__builtin_bit_cast(uint32_t, k) + 0x00400000u) & 0x7F800000u;
+    const float k2 = __builtin_bit_cast(float, k2_bits);
+    ratio = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
+        int, k * __builtin_bit_cast(float, 0x7F000000u - k2_bits))));
+    double w2sum = 0.0;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int c = 16 * t + n;
+      const bool cv = c < D1;
+      const int cc = cv ? c : 0;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int kk = KS * q + s;
+        float v = 0.0f;
+        if (kk < D0) v = s_w[kk * D1 + cc];
+        else if (kk == D0) v = s_w[oB1 + cc];
+        w1b[s][t] = cv ? v * kExp2Scale : 0.0f;
+      }
+      const float w2c = cv ? s_w[oW2 + cc] : 0.0f;
+      w2sum += (double)w2c;
+      w2g[t] = -2.0f * w2c * k2;
+    }
+    // sum over all hidden units in double, the same bits in every lane of a row of 16
+#pragma unroll
+    for (int msk = 1; msk < 16; msk <<= 1) w2sum += shfl_xor_d(w2sum, msk);
+    const double c0 = (w2sum - (double)s_w[oB2]) * (double)k2;
+    const float c0_hi = (float)c0, c0_lo = (float)(c0 - (double)c0_hi);
+    y_k = n == 0 ? k2 : 0.0f;
+    y_0 = n == 0 ? c0_hi : (n == 1 ? c0_lo : 0.0f);
+  }
+
+  __device__ __forceinline__ void zero_acc() {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      dacc[t][0] = f4{0.f, 0.f, 0.f, 0.f};
+      dacc[t][1] = f4{0.f, 0.f, 0.f, 0.f};
+      dw2s[t] = 0.0f;
+    }
+    dl = 0.0;
+  }
+
+  // rows past the end read as the last row (their gradient is masked to zero); any alignment
+  __device__ __forceinline__ void load_tile_safe(TileIn& ti, const StepCtx& cx, int row0, int n,
+                                                 int q) const {
+    const int last = cx.n - 1;
+    const int rowa = min(row0 + n, last);
+    const float* ra = cx.X + (size_t)rowa * D0;
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int k0 = KS * q + 2 * i;
+      const int kc = k0 < D0 ? k0 : D0 - 2;
+      f2 v = f2{ra[kc], ra[kc + 1]};
+      if (k0 >= D0) v = f2{k0 == D0 ? 1.0f : 0.0f, 0.0f};
+      ti.xa[i] = v;
+    }
+    const int f0 = 2 * n;
+    const int fc = f0 < D0 ? f0 : D0 - 2;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int rowb = min(row0 + 4 * q + j, last);
+      const float* rb = cx.X + (size_t)rowb * D0 + fc;
+      f2 v = f2{rb[0], rb[1]};
+      if (f0 >= D0) v = f2{f0 == D0 ? 1.0f : 0.0f, 0.0f};
+      ti.xb[j] = v;
+      ti.yv[j] = cx.y[rowb];
+    }
+  }
+
+  // ---- the four stages of a tile ----
+  // B: GEMM1, pre-activations (bias included through the constant-one feature)
+  __device__ __forceinline__ void gemm1(const f2 (&xa)[KP], f4 (&acc)[NT]) const {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[i][0], w1b[2 * i][t], acc[t], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[i][1], w1b[2 * i + 1][t], acc[t], 0, 0, 0);
+    }
+  }
+
+  // C: activation, layer-2 dot, per-row loss gradient, layer-2 weight gradient, the two GEMM2
+  // operands.  acc arrives as the exp2 argument t = -2 x / ln 2 of s = 1 / (1 + 2^t), tanh(x) = 2 s - 1
+  // (kernel_helpers.h:34-42 without its small-|x| identity branch, which changes the value by less
+  // than 1.5e-7), and leaves as s (1 - s) = (1 - tanh^2) / 4.  The factors g (per row) and 4 w2[c]
+  // (per hidden unit) of delta = (1 - h^2) w2[c] g (kernel_helpers.h:43, mcmc_step_ffma.h:323) are
+  // applied to the other GEMM2 operand (xg = g x_aug: 8 products per tile instead of 12) and once
+  // per step to the GEMM2 result.  The padded hidden units (zero weights: s = 1/2) carry 1/4, so the
+  // constant-one column of GEMM2 delivers sum(g) / 4 = db2 / 4 in row c = D1 for free.
+  template <int LIK, bool LAST, bool FULL>
+  __device__ __forceinline__ void pointwise(f4 (&acc)[NT], const f4& yv, const f2 (&xb)[4],
+                                            f2 (&xg)[4], const StepCtx& cx, const ModelConsts& mc,
+                                            int row0, int n, int q) {
+    float yh[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) yh[j] = __builtin_fmaf(yv[j], y_k, y_0);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float e = __builtin_amdgcn_exp2f(acc[t][j]);
+        const float sg = __builtin_amdgcn_rcpf(1.0f + e);
+        acc[t][j] = sg;
+        yh[j] = __builtin_fmaf(w2g[t], sg, yh[j]);
+      }
+    }
+    // (y - yhat - b2) k2 of the four rows 4 q + j, in bank j of one register; the loss gradient
+    // (Gaussian: that value itself, its factor k / k2 is applied to the sums once per step;
+    // Student-t: mcmc_step_ffma.h:293-301) is computed on that one register
+    const float rz = row16_reduce4(yh[0], yh[1], yh[2], yh[3]);
+    float gz = rz, dz = rz;
+    if (LIK == 0) {
+      dz = rz * ratio;
+      gz = dz * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(dz, dz, mc.df));
+    }
+    float g[4] = {row16_bcast<0>(gz), row16_bcast<1>(gz), row16_bcast<2>(gz), row16_bcast<3>(gz)};
+    if (!FULL) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) g[j] = row0 + 4 * q + j < cx.n ? g[j] : 0.0f;  // mcmc_step_ffma.h:301
+    }
+    if (LAST) {
+      const float d4[4] = {row16_bcast<0>(dz), row16_bcast<1>(dz), row16_bcast<2>(dz), row16_bcast<3>(dz)};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool valid = FULL || (row0 + 4 * q + j < cx.n);
+        if (n == 0 && valid) {
+          const float diff = LIK == 1 ? d4[j] * (ratio * mc.scale) : d4[j];
+          const int row = row0 + 4 * q + j;
+          const float lv = lik_value<LIK>(mc, diff);
+          const float prev = cx.ell_prev ? cx.ell_prev[row] : 0.0f;
+          if (cx.ell_new) cx.ell_new[row] = lv;
+          dl += (double)(lv - prev);
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float sg = acc[t][j];
+        dw2s[t] = __builtin_fmaf(g[j], sg, dw2s[t]);
+        acc[t][j] = __builtin_fmaf(-sg, sg, sg);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xg[j] = xb[j] * g[j];
+  }
+
+  // D: GEMM2, dacc += (s (1 - s))^T (g X_aug)
+  __device__ __forceinline__ void gemm2(const f4 (&dlt)[NT], const f2 (&xb)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        dacc[t][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(dlt[t][j], xb[j][0], dacc[t][0], 0, 0, 0);
+        dacc[t][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(dlt[t][j], xb[j][1], dacc[t][1], 0, 0, 0);
+      }
+    }
+  }
+
+  // Software-pipelined loop over full, aligned tiles [tb, te).  Iteration i issues the loads of tile
+  // i + 2, GEMM1 of tile i + 1, the pointwise work of tile i and GEMM2 of tile i - 1, all in one
+  // basic block, so the matrix pipe (42 MFMAs per tile) and the vector ALU (the pointwise work) run
+  // side by side inside one wave.  Lanes whose operand slot is the constant-one feature or padding
+  // read it from a small constant table through a per-lane pointer with stride zero, so no select
+  // sits between a load and its use.
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void fast_loop(const StepCtx& cx, const ModelConsts& mc, int tb, int te,
+                                            int n, int q) {
+    const AugTable<D0>* aug = aug_table<D0>();
+    const size_t tile_floats = (size_t)16 * D0;
+    // A operand: pairs 0 .. KP-2 are always real features; the last pair of lane group q = 3 is
+    // the (1, 0) constant
+    const float* pa = cx.X + (size_t)n * D0 + KS * q;
+    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
+    const float* pa_last0 = a_const ? aug->one : pa + (size_t)tb * tile_floats + 2 * (KP - 1);
+    const unsigned sa_last = a_const ? 0u : (unsigned)tile_floats;
+    // B operand of GEMM2: feature pair 2n, 2n+1 of rows 4q + j
+    const bool b_const = 2 * n >= D0;
+    const float* pb0 = b_const ? (2 * n == D0 ? aug->one : aug->zero)
+                               : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 2 * n;
+    const unsigned sb = b_const ? 0u : (unsigned)tile_floats;
+    const float* py = cx.y + 4 * q;
+
+    auto load = [&](TileIn& ti, int tile) {
+      const float* ra = pa + (size_t)tile * tile_floats;
+#pragma unroll
+      for (int i = 0; i < KP - 1; ++i) ti.xa[i] = *reinterpret_cast<const f2*>(ra + 2 * i);
+      const unsigned rel = (unsigned)(tile - tb);
+      ti.xa[KP - 1] = *reinterpret_cast<const f2*>(pa_last0 + (size_t)rel * sa_last);
+      const float* rb = pb0 + (size_t)rel * sb;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ti.xb[j] = *reinterpret_cast<const f2*>(rb + j * D0);
+      ti.yv = *reinterpret_cast<const f4*>(py + (size_t)tile * 16);
+    };
+
+    TileIn t0, t1, t2;  // tiles i, i + 1, i + 2
+    f4 acc_cur[NT], acc_nxt[NT], dlt_prev[NT];
+    f2 xb_prev[4];
+    load(t0, tb);
+    load(t1, tb + 1 < te ? tb + 1 : tb);
+    gemm1(t0.xa, acc_cur);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) dlt_prev[t] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xb_prev[j] = t0.xb[j];
+    for (int i = tb; i < te; ++i) {
+      load(t2, i + 2 < te ? i + 2 : te - 1);
+      gemm1(t1.xa, acc_nxt);                                       // tile i + 1
+      gemm2(dlt_prev, xb_prev);                                    // tile i - 1 (zero delta at i = tb)
+      f2 xg[4];
+      pointwise<LIK, LAST, true>(acc_cur, t0.yv, t0.xb, xg, cx, mc, i * 16, n, q);  // tile i
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        dlt_prev[t] = acc_cur[t];
+        acc_cur[t] = acc_nxt[t];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xb_prev[j] = xg[j];
+      t0 = t1;
+      t1 = t2;
+    }
+    gemm2(dlt_prev, xb_prev);  // tile te - 1
+  }
+
+  // Plain loop over full, aligned tiles [tb, te): loads one tile ahead, then GEMM1, pointwise work
+  // and GEMM2 of the current tile back to back.  Needs few registers, so more waves fit a SIMD and
+  // fill each other's dependency and memory stalls.
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void simple_loop(const StepCtx& cx, const ModelConsts& mc, int tb,
+                                              int te, int n, int q) {
+    const AugTable<D0>* aug = aug_table<D0>();
+    const size_t tile_floats = (size_t)16 * D0;
+    const float* pa = cx.X + (size_t)n * D0 + KS * q;
+    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
+    const float* pa_last0 = a_const ? aug->one : pa + (size_t)tb * tile_floats + 2 * (KP - 1);
+    const unsigned sa_last = a_const ? 0u : (unsigned)tile_floats;
+    const bool b_const = 2 * n >= D0;
+    const float* pb0 = b_const ? (2 * n == D0 ? aug->one : aug->zero)
+                               : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 2 * n;
+    const unsigned sb = b_const ? 0u : (unsigned)tile_floats;
+    const float* py = cx.y + 4 * q;
+    auto load = [&](TileIn& ti, int tile) {
+      const float* ra = pa + (size_t)tile * tile_floats;
+#pragma unroll
+      for (int i = 0; i < KP - 1; ++i) ti.xa[i] = *reinterpret_cast<const f2*>(ra + 2 * i);
+      const unsigned rel = (unsigned)(tile - tb);
+      ti.xa[KP - 1] = *reinterpret_cast<const f2*>(pa_last0 + (size_t)rel * sa_last);
+      const float* rb = pb0 + (size_t)rel * sb;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ti.xb[j] = *reinterpret_cast<const f2*>(rb + j * D0);
+      ti.yv = *reinterpret_cast<const f4*>(py + (size_t)tile * 16);
+    };
+    TileIn cur, nx1, nx2;  // loads run two tiles ahead of their use
+    load(cur, tb);
+    load(nx1, tb + 1 < te ? tb + 1 : te - 1);
+    for (int i = tb; i < te; ++i) {
+      load(nx2, i + 2 < te ? i + 2 : te - 1);
+      f4 acc[NT];
+      f2 xg[4];
+      gemm1(cur.xa, acc);
+      pointwise<LIK, LAST, true>(acc, cur.yv, cur.xb, xg, cx, mc, i * 16, n, q);
+      gemm2(acc, xg);
+      cur = nx1;
+      nx1 = nx2;
+    }
+  }
+
+  // ---- explicitly prefetched loop ----
+  // The compiler sinks ordinary loads of read-only data next to their first use, which undoes any
+  // prefetch written in the source.  Here the loads are issued by inline assembly, which it neither
+  // moves nor waits for, two tiles ahead of their use into three rotating register sets, and the
+  // waits are explicit: s_waitcnt vmcnt(14) leaves the two newer tiles (7 loads each) in flight.
+  // Memory operations the compiler adds on its own (the last step's log-likelihood rows, spills)
+  // only make these waits more conservative, never too short: vmcnt counts every outstanding
+  // operation in issue order.
+  struct TileRaw {
+    f4 xa01;   // GEMM1 operand, k-pairs 0 and 1
+    f2 xa2;    // k-pair 2 (the (1, 0) constant in lane group q = 3)
+    f2 xb[4];  // GEMM2 operand
+    f4 yv;
+  };
+  template <int N>
+  static __device__ __forceinline__ void wait_tile(TileRaw& t) {
+    asm volatile("s_waitcnt vmcnt(%[cnt])"
+                 : "+v"(t.xa01), "+v"(t.xa2), "+v"(t.xb[0]), "+v"(t.xb[1]), "+v"(t.xb[2]), "+v"(t.xb[3]),
+                   "+v"(t.yv)
+                 : [cnt] "n"(N)
+                 : "memory");
+  }
+
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void prefetch_loop(const StepCtx& cx, const ModelConsts& mc, int tb,
+                                                int te, int n, int q) {
+    static_assert(KP == 3, "register sets are laid out for three k-pairs");
+    // Every load is  base (wave-uniform, in SGPRs, advanced by scalar instructions)  +  a 32-bit
+    // per-lane offset that never changes: no vector instruction is spent on addresses.  Lanes whose
+    // operand slot is the constant-one feature or padding do not load at all: their registers are
+    // set once, below, and the loads of those slots run with these lanes masked out of EXEC.
+    const unsigned oa = (unsigned)((n * D0 + KS * q) * 4);
+    const unsigned ol = oa + 2 * (KP - 1) * 4;
+    const unsigned ob = (unsigned)(((4 * q) * D0 + 2 * n) * 4);
+    const unsigned oy = (unsigned)(4 * q * 4);
+    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
+    const bool b_const = 2 * n >= D0;
+    const unsigned long long mask_a = __builtin_amdgcn_ballot_w64(!a_const);
+    const unsigned long long mask_b = __builtin_amdgcn_ballot_w64(!b_const);
+    const f2 const_a = f2{1.0f, 0.0f};
+    const f2 const_b = f2{2 * n == D0 ? 1.0f : 0.0f, 0.0f};
+    int nxt = tb;  // tiles are issued in order, one call each; past the last tile the base stays
+    auto issue = [&](TileRaw& t) {  // exactly 7 loads
+      const int tile = nxt < te ? nxt : te - 1;
+      ++nxt;
+      const float* bx = cx.X + (size_t)tile * (16 * D0);
+      const float* by = cx.y + (size_t)tile * 16;
+      // One block for the seven loads.  The leading s_nop gives the five wait states a memory
+      // instruction needs after a VALU instruction wrote one of its SGPR operands (the compiler
+      // reloads spilled SGPRs with v_readlane and does not see the loads inside the assembly, so it
+      // would not insert them itself).  EXEC is saved on entry and put back.  The pure outputs are
+      // early-clobber: a returning load must not land in a register that still holds an offset of a
+      // load not yet issued.
+      unsigned long long exec_save;
+      asm volatile(
+          "s_mov_b64 %[sv], exec\n\t"
+          "s_nop 3\n\t"
+          "global_load_dwordx4 %[xa01], %[oa], %[bx]\n\t"
+          "s_and_b64 exec, %[sv], %[ma]\n\t"
+          "global_load_dwordx2 %[xa2], %[ol], %[bx]\n\t"
+          "s_and_b64 exec, %[sv], %[mb]\n\t"
+          "global_load_dwordx2 %[xb0], %[ob], %[bx]\n\t"
+          "global_load_dwordx2 %[xb1], %[ob], %[bx] offset:%[r1]\n\t"
+          "global_load_dwordx2 %[xb2], %[ob], %[bx] offset:%[r2]\n\t"
+          "global_load_dwordx2 %[xb3], %[ob], %[bx] offset:%[r3]\n\t"
+          "s_mov_b64 exec, %[sv]\n\t"
+          "global_load_dwordx4 %[yv], %[oy], %[by]"
+          : [xa01] "=&v"(t.xa01), [xa2] "+v"(t.xa2), [xb0] "+v"(t.xb[0]), [xb1] "+v"(t.xb[1]),
+            [xb2] "+v"(t.xb[2]), [xb3] "+v"(t.xb[3]), [yv] "=&v"(t.yv), [sv] "=&s"(exec_save)
+          : [oa] "v"(oa), [ol] "v"(ol), [ob] "v"(ob), [oy] "v"(oy), [bx] "s"(bx), [by] "s"(by),
+            [ma] "s"(mask_a), [mb] "s"(mask_b), [r1] "n"(D0 * 4), [r2] "n"(2 * D0 * 4),
+            [r3] "n"(3 * D0 * 4)
+          : "memory", "scc");
+    };
+    auto preset = [&](TileRaw& t) {
+      t.xa2 = const_a;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t.xb[j] = const_b;
+    };
+    auto compute = [&](TileRaw& t, int tile) {
+      const f2 xa[KP] = {f2{t.xa01[0], t.xa01[1]}, f2{t.xa01[2], t.xa01[3]}, t.xa2};
+      f4 acc[NT];
+      f2 xg[4];
+      gemm1(xa, acc);
+      pointwise<LIK, LAST, true>(acc, t.yv, t.xb, xg, cx, mc, tile * 16, n, q);
+      // keep the stages apart: left to itself the scheduler may feed each GEMM2 operand to its
+      // MFMAs the moment it is computed, which puts two wait states in front of every other MFMA
+      __builtin_amdgcn_sched_barrier(0);
+      gemm2(acc, xg);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    TileRaw A, B, C;
+    preset(A);
+    preset(B);
+    preset(C);
+    issue(A);
+    issue(B);
+    // steady state: three tiles per trip, every issue and every wait unconditional.
+    // Two waves share a SIMD, and the matrix and vector instructions of both go through one FP32
+    // pipe: it stays busy only while both waves have work (each fills the dependency stalls of the
+    // other).  The hardware favours the older wave, which would finish its tiles long before the
+    // younger one and leave it to run alone, stalls exposed.  So every trip a wave publishes its
+    // tile count in LDS, reads its partner's, and takes the higher priority while it is behind.
+    int i = tb;
+    const bool balance = cx.progress != nullptr;
+    for (; i + 3 <= te; i += 3) {
+      issue(C);
+      wait_tile<14>(A);
+      compute(A, i);
+      issue(A);
+      wait_tile<14>(B);
+      compute(B, i + 1);
+      issue(B);
+      wait_tile<14>(C);
+      compute(C, i + 2);
+      if (balance) {
+        // all operands are wave-uniform: the registers live only across these three instructions
+        const unsigned my_slot = (unsigned)(size_t)(cx.progress + cx.wave);  // LDS byte addresses
+        const unsigned other_slot = (unsigned)(size_t)(cx.progress + cx.partner);
+        const int done = i + 3 - tb;
+        int other;
+        asm volatile("ds_write_b32 %1, %2\n\tds_read_b32 %0, %3\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(other)
+                     : "v"(my_slot), "v"(done), "v"(other_slot)
+                     : "memory");
+        if (__builtin_amdgcn_readfirstlane(other) > done) __builtin_amdgcn_s_setprio(2);
+        else __builtin_amdgcn_s_setprio(0);
+      }
+    }
+    if (balance) __builtin_amdgcn_s_setprio(0);
+    // no register of a set may be used or reused before its last load has landed
+    wait_tile<0>(A);
+    wait_tile<0>(B);
+    wait_tile<0>(C);
+    // the one or two tiles left over: A and B hold them (issued at the end of the last trip)
+    if (i < te) compute(A, i);
+    if (i + 1 < te) compute(B, i + 1);
+  }
+
+  template <int LIK, bool LAST>
+  __device__ __forceinline__ void run_tiles(const StepCtx& cx, const ModelConsts& mc) {
+    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    const int tb = cx.tile_begin, te = cx.tile_end;
+    int fast_end = tb;
+    if (cx.x_vec_ok && cx.y_vec_ok) fast_end = min(te, cx.n / 16);
+    if (fast_end > tb) {
+      if (PIPE == 1) fast_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
+      else if (PIPE == 2) prefetch_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
+      else simple_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
+    }
+    // ragged tail tile, or unaligned caller buffers: one tile at a time
+    for (int tile = max(tb, fast_end); tile < te; ++tile) {
+      TileIn ti;
+      f4 acc[NT];
+      load_tile_safe(ti, cx, tile * 16, n, q);
+      f2 xg[4];
+      gemm1(ti.xa, acc);
+      pointwise<LIK, LAST, false>(acc, ti.yv, ti.xb, xg, cx, mc, tile * 16, n, q);
+      gemm2(acc, xg);
+    }
+  }
+
+  // this wave's partial sums -> its LDS slot, indexed by canonical parameter number; the factors
+  // 4 w2[c] left out of the GEMM2 operand and k / k2 left out of g are applied here
+  template <int LIK>
+  __device__ __forceinline__ void write_partials(float* slot, const float* s_w) {
+    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    static_assert(D1 % 16 != 0, "db2 rides in the first padded hidden unit");
+    const float gr = LIK == 1 ? ratio : 1.0f;
+    const float gr4 = 4.0f * gr;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int f = 2 * n + u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int c = 16 * t + 4 * q + j;
+          if (c < D1) {
+            const float v = dacc[t][u][j] * (gr4 * s_w[oW2 + c]);
+            if (f < D0) slot[f * D1 + c] = v;
+            else if (f == D0) slot[oB1 + c] = v;
+          } else if (c == D1 && f == D0) {
+            slot[oB2] = gr4 * dacc[t][u][j];  // sum of g over this wave's rows
+          }
+        }
+      }
+      // dw2 = sum_rows g h = 2 (sum_rows g s - sum_rows g / 2); the second sum is what the first padded
+      // hidden unit (lane n = D1 % 16 of the last hidden tile, s = 1/2) has accumulated; the four row
+      // groups q in a fixed order
+      const float half_gsum = dpp_move<0x150 + D1 % 16>(dw2s[NT - 1]);  // row_newbcast
+      float v = 2.0f * (dw2s[t] - half_gsum) * gr;
+      v += __shfl_xor(v, 16);
+      v += __shfl_xor(v, 32);
+      const int c = 16 * t + n;
+      if (q == 0 && c < D1) slot[oW2 + c] = v;
+    }
+    double d = dl;  // held by lanes n == 0
+    d += shfl_xor_d(d, 16);
+    d += shfl_xor_d(d, 32);
+    if (lane == 0) {
+      const uint64_t bits = double_to_bits(d);
+      slot[P_AL] = __builtin_bit_cast(float, (uint32_t)bits);
+      slot[P_AL + 1] = __builtin_bit_cast(float, (uint32_t)(bits >> 32));
+    }
+  }
+};
+
+}  // namespace bnn

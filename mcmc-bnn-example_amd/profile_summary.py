@@ -22,6 +22,13 @@ def counter_totals(path, kernel_substr):
     return agg
 
 
+def bench_json(path):
+    try:
+        return json.loads(open(path).read().strip().splitlines()[-1])
+    except Exception:  # noqa: BLE001
+        return None
+
+
 def main(out):
     lines = []
     stats = find(os.path.join(out, "trace"), "*kernel_stats.csv")
@@ -36,21 +43,22 @@ def main(out):
     if kt:
         durs = [(int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e6
                 for r in csv.DictReader(open(kt)) if "hmc_kernel" in r["Kernel_Name"]]
-        lines.append("hmc_kernel dispatch durations, ms (the first is the bootstrap evaluation, then one per "
-                     "launch of transitions): " + ", ".join("%.3f" % d for d in durs))
-        big = [d for d in durs if d > 0.5 * max(durs)]
-        if big:
-            lines.append("average over the %d full-size launches: %.3f ms" % (len(big), sum(big) / len(big)))
-    bj = os.path.join(out, "bench_trace.json")
-    if os.path.exists(bj):
-        try:
-            d = json.loads(open(bj).read().strip().splitlines()[-1])
-            lines.append("bench.py under the tracer: %.0f grad-evals/s, roofline frac %.3f, %.3f ms per launch "
-                         "(HIP events), %d launches" % (d["value"], d["roofline"]["frac"],
-                                                        d["roofline"]["ms_per_launch"], d["roofline"]["launches"]))
-        except Exception as e:  # noqa: BLE001
-            lines.append("bench json unreadable: %r" % e)
-    scale = {}
+        # launches of transitions take tens of milliseconds and more; the bootstrap and state
+        # evaluations that precede them well under one
+        trans = [d for d in durs if d > 5.0]
+        lines.append("hmc_kernel dispatches: %d evaluation launches (%.3f ms in all), %d launches of "
+                     "transitions: %s ms" % (len(durs) - len(trans), sum(durs) - sum(trans), len(trans),
+                                             ", ".join("%.1f" % d for d in trans)))
+        if trans:
+            lines.append("average over the %d launches of transitions: %.3f ms" % (
+                len(trans), sum(trans) / len(trans)))
+    d = bench_json(os.path.join(out, "bench_trace.json"))
+    if d:
+        lines.append("bench.py under the tracer: %.0f grad-evals/s, roofline frac %.3f, %.3f ms per launch "
+                     "(HIP events over the timed region), %d launches" % (
+                         d["value"], d["roofline"]["frac"], d["roofline"]["ms_per_launch"],
+                         d["roofline"]["launches"]))
+    scale, total_bytes, evals = {}, 0.0, None
     for c in ("FETCH_SIZE", "WRITE_SIZE"):
         cp = find(os.path.join(out, "copy_" + c), "*counter_collection.csv")
         kp = find(os.path.join(out, "pmc_" + c), "*counter_collection.csv")
@@ -62,10 +70,29 @@ def main(out):
                          % (c, v, scale[c]))
         if kp:
             tot = counter_totals(kp, "hmc_kernel")
-            big = sorted(tot.items(), key=lambda kv: -kv[1][c])[:3]
+            allv = sum(v[c] for v in tot.values())
+            big = sorted(tot.items(), key=lambda kv: -kv[1][c])[:2]
             for disp, v in big:
-                lines.append("%s, hmc_kernel dispatch %s: %.0f counted = %.1f MiB after scaling" % (
+                lines.append("%s, largest hmc_kernel dispatch %s: %.0f counted = %.1f MiB after scaling" % (
                     c, disp, v[c], v[c] * scale.get(c, 1.0) / 1024.0))
+            lines.append("%s, all %d hmc_kernel dispatches: %.0f counted = %.1f MiB after scaling" % (
+                c, len(tot), allv, allv * scale.get(c, 1.0) / 1024.0))
+            total_bytes += allv * scale.get(c, 1.0) * 1024.0
+            b = bench_json(os.path.join(out, "bench_%s.json" % c))
+            if b:
+                evals = b["roofline"]["grad_evals_per_launch"] * b["roofline"]["launches"] * (
+                    b["steps"] + b["warmup"]) / b["steps"]
+    if total_bytes and evals:
+        lines.append("HBM traffic: %.4g bytes over %.0f gradient evaluations = %.0f bytes per evaluation" % (
+            total_bytes, evals, total_bytes / evals))
+        key = "hmc_kernel_wide_64x128" if d and "64->128" in d["config"]["workload"] else (
+            "hmc_kernel_%s_22x40" % (d["config"]["layer"] if d else "mfma"))
+        json.dump({key: {"bytes_per_grad_eval": total_bytes / evals,
+                         "source": "rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over every trajectory-kernel "
+                                   "dispatch of one bench.py run, each scaled by the same counter on a 1 GiB "
+                                   "copy kernel",
+                         "cus_per_chain": d["config"]["cus_per_chain"] if d else None}},
+                  open(os.path.join(out, "traffic.json"), "w"), indent=1)
     sq = find(os.path.join(out, "pmc_SQ"), "*counter_collection.csv")
     if sq:
         tot = counter_totals(sq, "hmc_kernel")

@@ -67,11 +67,13 @@ def test_20_transitions_from_the_adapted_state_at_full_size(config0_chain, orc):
     10), 20 transitions of 1000 leapfrog steps on the GPU and on the oracle, same RNG counters.
 
     The log accept ratio is a sum over 58368 rows at the end of a 1000-step trajectory; FP32 rounding
-    differences of the gradient (1e-7 relative) grow along it, and the two implementations were
-    measured to differ by up to 0.062 in it.  Decisions must therefore agree wherever the uniform is
-    further than MARGIN = 0.15 from the oracle's ratio; how many transitions fall inside the margin is
-    reported, and at most two of the 20 may disagree in all."""
-    MARGIN = 0.15
+    differences of the gradient (1e-7 relative) grow along it, the more the larger the energy error of
+    the trajectory is.  Over several builds of the kernel (each takes the burn-in a different way, so
+    each starts this leg from another state) the two implementations differed by up to 0.15 in it where
+    it is of order 1 and by up to 0.19 where it is of order 6, and never in a decision.  The tolerance
+    is TOL = 0.25 + 0.1 |log alpha|: the two values must agree to TOL, decisions must agree wherever the
+    uniform is further than TOL from the oracle's ratio, how many transitions fall inside that margin
+    is reported, and at most two of the 20 may disagree in all."""
     c = config0_chain
     s, st = c["s"], c["state"]
     assert st["transitions_done"] == 100
@@ -83,16 +85,20 @@ def test_20_transitions_from_the_adapted_state_at_full_size(config0_chain, orc):
     lu = np.array([orc.log_uniform(0, 0, 100 + k) for k in range(20)])
     la_gpu, la_ref = tr["log_acpt"][100:120], ref["log_acpt"]
     acc_gpu, acc_ref = tr["accept"][100:120], ref["accept"]
-    clear = np.abs(lu - la_ref) > MARGIN
-    say("adapted leg: %d of 20 transitions inside the margin; max |log alpha gpu - oracle| = %.4f; "
-        "accepted gpu %d, oracle %d" % ((~clear).sum(), np.abs(la_gpu - la_ref).max(), acc_gpu.sum(),
+    tol = 0.25 + 0.1 * np.abs(la_ref)
+    clear = np.abs(lu - la_ref) > tol
+    say("adapted leg: %d of 20 transitions inside the margin; max |log alpha gpu - oracle| / tolerance = %.2f; "
+        "accepted gpu %d, oracle %d" % ((~clear).sum(), (np.abs(la_gpu - la_ref) / tol).max(), acc_gpu.sum(),
                                          acc_ref.sum()))
+    for k in range(20):
+        say("  t=%d log u %.4f  log alpha gpu %.4f oracle %.4f  accept %d %d" % (
+            100 + k, lu[k], la_gpu[k], la_ref[k], acc_gpu[k], acc_ref[k]))
     assert np.all(np.isfinite(la_gpu)) and np.all(np.isfinite(la_ref))
     assert np.array_equal(acc_gpu[clear], acc_ref[clear])
     assert clear.sum() >= 12, "too few transitions outside the margin to say anything"
     assert (acc_gpu != acc_ref).sum() <= 2
-    assert np.abs(la_gpu - la_ref).max() < MARGIN
-    assert 0 < acc_ref.sum() < 20 or acc_ref.sum() == 20      # an adapted chain accepts most of them
+    assert np.all(np.abs(la_gpu - la_ref) < tol)
+    assert acc_ref.sum() >= 3                                 # an adapted chain does accept
     # the step size no longer changes after the burn-in
     assert np.all(tr["eps"][100:120] == np.float32(st["eps"]))
 
