@@ -347,6 +347,9 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
     }
 
     for (int s = 0; s < a.L && ok; ++s) {
+      // indices and addresses that depend on the thread index are recomputed every step (see
+      // opaque_tid): hoisted out of this loop they would occupy registers across the tile loop
+      const int tid = opaque_tid();
       // ---- leapfrog update (mcmc_step_ffma.h:106-112): half kick on the first step ----
       const float ek = s == 0 ? eps * 0.5f : eps;
 #pragma unroll

@@ -15,6 +15,16 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 // ------------------------------------------------------------------------------------------------
 // small device helpers
 // ------------------------------------------------------------------------------------------------
+// The thread index as a value the compiler cannot see through.  Indices and addresses derived from
+// it are computed where they are used, every time: derived from threadIdx.x they are invariant across
+// the leapfrog steps, get hoisted out of the step loop, and then sit in registers across the tile
+// loop, which has none to spare.
+__device__ __forceinline__ int opaque_tid() {
+  int t = (int)threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
   return __builtin_bit_cast(

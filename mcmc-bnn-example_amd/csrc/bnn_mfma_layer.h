@@ -90,7 +90,7 @@ struct MfmaLayer {
 
   template <int LIK>
   __device__ __forceinline__ void load_weights(const float* s_w, const ModelConsts& mc) {
-    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    const int lane = opaque_tid() & 63, n = lane & 15, q = lane >> 4;
     const float k = LIK == 1 ? mc.scale_recp * mc.scale_recp : mc.scale_recp;
     // the power of two next to k, and its reciprocal
     const uint32_t k2_bits = (__builtin_bit_cast(uint32_t, k) + 0x00400000u) & 0x7F800000u;
@@ -505,7 +505,7 @@ struct MfmaLayer {
 
   template <int LIK, bool LAST>
   __device__ __forceinline__ void run_tiles(const StepCtx& cx, const ModelConsts& mc) {
-    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    const int lane = opaque_tid() & 63, n = lane & 15, q = lane >> 4;
     const int tb = cx.tile_begin, te = cx.tile_end;
     int fast_end = tb;
     if (cx.x_vec_ok && cx.y_vec_ok) fast_end = min(te, cx.n / 16);
@@ -530,7 +530,7 @@ struct MfmaLayer {
   // 4 w2[c] left out of the GEMM2 operand and k / k2 left out of g are applied here
   template <int LIK>
   __device__ __forceinline__ void write_partials(float* slot, const float* s_w) {
-    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    const int lane = opaque_tid() & 63, n = lane & 15, q = lane >> 4;
     static_assert(D1 % 16 != 0, "db2 rides in the first padded hidden unit");
     const float gr = LIK == 1 ? ratio : 1.0f;
     const float gr4 = 4.0f * gr;
