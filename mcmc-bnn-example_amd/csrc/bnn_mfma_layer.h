@@ -32,19 +32,25 @@ __device__ __forceinline__ const AugTable<22>* aug_table<22>() {
 }
 
 // ================================================================================================
-// MFMA layer: both contractions on v_mfma_f32_16x16x4_f32.
+// MFMA layer: GEMM1 and most of GEMM2 on v_mfma_f32_16x16x4_f32, the rest of GEMM2 on
+// v_mfma_f32_4x4x1_16B_f32 (same flops per cycle, but sixteen independent 4x4 outer products: no
+// padding of the seven feature columns that a second 16-wide tile would leave half empty).
 //
-// Lane l = 16 q + n (q = 0..3, n = 0..15).  A 16-row tile is processed as
-//   GEMM1  A = X_aug tile  [16 rows x K]   lane (n, q) holds row n, k = KS q + s      (s < KS)
-//          B = W1_aug      [K x 16 c]      lane (n, q) holds k = KS q + s, c = 16 t + n
-//          C = pre-act     [16 rows x 16 c] lane (n, q) holds rows 4 q + j, c = 16 t + n
-//   GEMM2  A = delta^T     [16 c x 4 rows]  = C layout of GEMM1 reused as is (k-step j <-> rows
-//                                             4 q + j): no shuffle between the two GEMMs
-//          B = X_aug tile  [4 rows x 16 f]  lane (n, q) holds row 4 q + j, features 2 n + u
-//          C = dW1_aug^T   [16 c x 16 f]    lane (n, q) holds c = 16 t + 4 q + j', f = 2 n + u
+// Lane l = 16 q + n (q = 0..3, n = 0..15; n = 4 cb + jj).  A 16-row tile is processed as
+//   GEMM1   A = X_aug tile  [16 rows x K]    lane (n, q) holds row n, k = KS q + s      (s < KS)
+//           B = W1_aug      [K x 16 c]       lane (n, q) holds k = KS q + s, c = 16 t + n
+//           C = pre-act     [16 rows x 16 c] lane (n, q) holds rows 4 q + j, c = 16 t + n
+//   GEMM2e  A = delta^T     [16 c x 4 rows]  = C layout of GEMM1 reused as is (k-step j <-> rows
+//                                              4 q + j): no shuffle between the two GEMMs
+//           B = X tile      [4 rows x 16 f]  lane (n, q) holds row 4 q + j, feature n      (f < 16)
+//           C = dW1^T       [16 c x 16 f]    lane (n, q) holds c = 16 t + 4 q + i, f = n
+//   GEMM2f  sixteen blocks b = 4 q + cb per instruction, one instruction per (t, j, fb):
+//           A block = delta of row 4 q + j, c = 16 t + 4 cb + i     (the same register as above)
+//           B block = X_aug of row 4 q + j, f = 16 + 2 jj + fb      (lane (n, q), any cb)
+//           D block = dW1_aug^T partial of row group q: vgpr i, lane (n, q): c = 16 t + 4 cb + i,
+//                     f = 16 + 2 jj + fb; the four row groups are added once per step
 // X_aug appends a constant-one feature (index D0) so that b1 rides in GEMM1 and db1 falls out of
-// GEMM2; the contraction index of GEMM1 and the feature index of GEMM2 are permuted so that every
-// lane reads contiguous floats of a row.
+// GEMM2; the contraction index of GEMM1 is permuted so that every lane reads contiguous floats.
 // ================================================================================================
 template <int D0, int D1, int PIPE>
 struct MfmaLayer {
@@ -53,7 +59,7 @@ struct MfmaLayer {
   static_assert(KS % 2 == 0, "k-steps are read in pairs");
   static constexpr int KP = KS / 2;
   static constexpr int NT = (D1 + 15) / 16;  // hidden tiles
-  static_assert(D0 + 1 <= 32, "one feature-pair tile");
+  static_assert(D0 > 16 && D0 + 2 <= 24, "features 16 .. D0 + 1 go through the 4x4 blocks");
   static constexpr int oB1 = D0 * D1, oW2 = oB1 + D1, oB2 = oW2 + D1, P = oB2 + 1;
   static constexpr int P_AL = (P + 3) / 4 * 4;
 
@@ -68,11 +74,13 @@ struct MfmaLayer {
                        // keeps the coefficients exact: the dot cancels from terms of size |w2| k to a
                        // residual thousands of times smaller, and a rounding error in a coefficient
                        // would be the same in every row and add up over the rows instead of averaging out
-  float y_k;           // k2 in lane n == 0, else 0
+  float y_k[4];        // y_k[j]: k2 in lane n == j, else 0 (lane n < 4 holds the target of row 4 q + n)
   float y_0;           // the constant part of the dot, (sum_c w2[c] - b2) k2, computed in double and
-                       // split over lanes n == 0 (leading part) and n == 1 (remainder)
+                       // split over lanes n == 4 (leading part) and n == 5 (remainder)
   float ratio;         // k / k2 (exact)
-  f4 dacc[NT][2];      // sum over rows of s (1 - s) g' x_aug, g' = g k2 / k (Gaussian) or g (Student-t)
+  // sums over rows of s (1 - s) g' x_aug, g' = g k2 / k (Gaussian) or g (Student-t):
+  f4 dacc_e[NT];       //   features 0 .. 15
+  f4 dacc_f[NT][2];    //   features 16 .. D0 + 1, partial over the rows of row group q
   float dw2s[NT];      // sum over rows of g' s
                        // (in the lanes of the padded hidden units, where s is exactly 1/2, this is half the
                        // sum over rows of g', added in the very order of the other lanes' sums: dw2 =
@@ -81,9 +89,10 @@ struct MfmaLayer {
   double dl;
 
   struct TileIn {
-    f2 xa[KP];
-    f2 xb[4];
-    f4 yv;
+    f2 xa[KP];   // GEMM1 operand
+    float xe[4]; // GEMM2e operand: feature n of rows 4 q + j
+    f2 xf[4];    // GEMM2f operand: features 16 + 2 jj, 17 + 2 jj of rows 4 q + j
+    float y1;    // target of row 4 q + (n & 3)
   };
 
   static constexpr float kExp2Scale = -2.88539008177792681472f;  // -2 / ln 2, kernel_helpers.h:37
@@ -120,19 +129,25 @@ struct MfmaLayer {
     for (int msk = 1; msk < 16; msk <<= 1) w2sum += shfl_xor_d(w2sum, msk);
     const double c0 = (w2sum - (double)s_w[oB2]) * (double)k2;
     const float c0_hi = (float)c0, c0_lo = (float)(c0 - (double)c0_hi);
-    y_k = n == 0 ? k2 : 0.0f;
-    y_0 = n == 0 ? c0_hi : (n == 1 ? c0_lo : 0.0f);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) y_k[j] = n == j ? k2 : 0.0f;
+    y_0 = n == 4 ? c0_hi : (n == 5 ? c0_lo : 0.0f);
   }
 
   __device__ __forceinline__ void zero_acc() {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      dacc[t][0] = f4{0.f, 0.f, 0.f, 0.f};
-      dacc[t][1] = f4{0.f, 0.f, 0.f, 0.f};
+      dacc_e[t] = f4{0.f, 0.f, 0.f, 0.f};
+      dacc_f[t][0] = f4{0.f, 0.f, 0.f, 0.f};
+      dacc_f[t][1] = f4{0.f, 0.f, 0.f, 0.f};
       dw2s[t] = 0.0f;
     }
     dl = 0.0;
   }
+
+  // the constant GEMM2f operand of lanes whose feature pair starts at or beyond D0: (1, 0) for the
+  // appended constant-one feature, else (0, 0)
+  static __device__ __forceinline__ f2 const_f(int jj) { return f2{16 + 2 * jj == D0 ? 1.0f : 0.0f, 0.0f}; }
 
   // rows past the end read as the last row (their gradient is masked to zero); any alignment
   __device__ __forceinline__ void load_tile_safe(TileIn& ti, const StepCtx& cx, int row0, int n,
@@ -148,20 +163,68 @@ struct MfmaLayer {
       if (k0 >= D0) v = f2{k0 == D0 ? 1.0f : 0.0f, 0.0f};
       ti.xa[i] = v;
     }
-    const int f0 = 2 * n;
+    const int jj = n & 3;
+    const int f0 = 16 + 2 * jj;
     const int fc = f0 < D0 ? f0 : D0 - 2;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int rowb = min(row0 + 4 * q + j, last);
-      const float* rb = cx.X + (size_t)rowb * D0 + fc;
-      f2 v = f2{rb[0], rb[1]};
-      if (f0 >= D0) v = f2{f0 == D0 ? 1.0f : 0.0f, 0.0f};
-      ti.xb[j] = v;
-      ti.yv[j] = cx.y[rowb];
+      const float* rb = cx.X + (size_t)rowb * D0;
+      ti.xe[j] = rb[n];
+      ti.xf[j] = f0 < D0 ? f2{rb[fc], rb[fc + 1]} : const_f(jj);
     }
+    ti.y1 = cx.y[min(row0 + 4 * q + jj, last)];
   }
 
-  // ---- the four stages of a tile ----
+  // ordinary loads of a full, aligned tile through per-lane pointers (the plain and the software-
+  // pipelined loop).  Lanes whose operand slot is the constant-one feature or padding read it from a
+  // small constant table through a pointer with stride zero, so no select sits between a load and its use.
+  struct PlainPtrs {
+    const float* pa;        // row n, k = KS q of tile 0
+    const float* pa_last0;  // last k-pair: real data, or the (1, 0) constant in lane group q = 3
+    unsigned sa_last;
+    const float* pe;        // rows 4 q + j, feature n
+    const float* pf0;       // rows 4 q + j, features 16 + 2 jj ..: real data or constants
+    unsigned sf;
+    const float* py;        // row 4 q + jj
+    int tb;
+  };
+  __device__ __forceinline__ PlainPtrs plain_ptrs(const StepCtx& cx, int tb, int n, int q) const {
+    const AugTable<D0>* aug = aug_table<D0>();
+    const size_t tile_floats = (size_t)16 * D0;
+    PlainPtrs p;
+    p.tb = tb;
+    p.pa = cx.X + (size_t)n * D0 + KS * q;
+    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
+    p.pa_last0 = a_const ? aug->one : p.pa + (size_t)tb * tile_floats + 2 * (KP - 1);
+    p.sa_last = a_const ? 0u : (unsigned)tile_floats;
+    p.pe = cx.X + (size_t)(4 * q) * D0 + n;
+    const int jj = n & 3;
+    const bool f_const = 16 + 2 * jj >= D0;
+    p.pf0 = f_const ? (16 + 2 * jj == D0 ? aug->one : aug->zero)
+                    : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 16 + 2 * jj;
+    p.sf = f_const ? 0u : (unsigned)tile_floats;
+    p.py = cx.y + 4 * q + jj;
+    return p;
+  }
+  __device__ __forceinline__ void load_plain(TileIn& ti, const PlainPtrs& p, int tile) const {
+    const size_t tile_floats = (size_t)16 * D0;
+    const float* ra = p.pa + (size_t)tile * tile_floats;
+#pragma unroll
+    for (int i = 0; i < KP - 1; ++i) ti.xa[i] = *reinterpret_cast<const f2*>(ra + 2 * i);
+    const unsigned rel = (unsigned)(tile - p.tb);
+    ti.xa[KP - 1] = *reinterpret_cast<const f2*>(p.pa_last0 + (size_t)rel * p.sa_last);
+    const float* re = p.pe + (size_t)tile * tile_floats;
+    const float* rf = p.pf0 + (size_t)rel * p.sf;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      ti.xe[j] = re[j * D0];
+      ti.xf[j] = *reinterpret_cast<const f2*>(rf + j * D0);
+    }
+    ti.y1 = p.py[(size_t)tile * 16];
+  }
+
+  // ---- the stages of a tile ----
   // B: GEMM1, pre-activations (bias included through the constant-one feature)
   __device__ __forceinline__ void gemm1(const f2 (&xa)[KP], f4 (&acc)[NT]) const {
 #pragma unroll
@@ -177,21 +240,21 @@ struct MfmaLayer {
     }
   }
 
-  // C: activation, layer-2 dot, per-row loss gradient, layer-2 weight gradient, the two GEMM2
+  // C: activation, layer-2 dot, per-row loss gradient, layer-2 weight gradient, the GEMM2
   // operands.  acc arrives as the exp2 argument t = -2 x / ln 2 of s = 1 / (1 + 2^t), tanh(x) = 2 s - 1
   // (kernel_helpers.h:34-42 without its small-|x| identity branch, which changes the value by less
   // than 1.5e-7), and leaves as s (1 - s) = (1 - tanh^2) / 4.  The factors g (per row) and 4 w2[c]
   // (per hidden unit) of delta = (1 - h^2) w2[c] g (kernel_helpers.h:43, mcmc_step_ffma.h:323) are
-  // applied to the other GEMM2 operand (xg = g x_aug: 8 products per tile instead of 12) and once
-  // per step to the GEMM2 result.  The padded hidden units (zero weights: s = 1/2) carry 1/4, so the
-  // constant-one column of GEMM2 delivers sum(g) / 4 = db2 / 4 in row c = D1 for free.
+  // applied to the other GEMM2 operand (g x_aug: 12 products per tile) and once per step to the GEMM2
+  // result.  The padded hidden units (zero weights: s = 1/2) carry 1/4, so the constant-one column
+  // of GEMM2 delivers sum(g) / 4 = db2 / 4 in row c = D1 for free.
   template <int LIK, bool LAST, bool FULL>
-  __device__ __forceinline__ void pointwise(f4 (&acc)[NT], const f4& yv, const f2 (&xb)[4],
-                                            f2 (&xg)[4], const StepCtx& cx, const ModelConsts& mc,
-                                            int row0, int n, int q) {
+  __device__ __forceinline__ void pointwise(f4 (&acc)[NT], const TileIn& ti, float (&ge)[4], f2 (&gf)[4],
+                                            const StepCtx& cx, const ModelConsts& mc, int row0, int n,
+                                            int q) {
     float yh[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) yh[j] = __builtin_fmaf(yv[j], y_k, y_0);
+    for (int j = 0; j < 4; ++j) yh[j] = __builtin_fmaf(ti.y1, y_k[j], y_0);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -241,124 +304,92 @@ struct MfmaLayer {
       }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) xg[j] = xb[j] * g[j];
+    for (int j = 0; j < 4; ++j) {
+      ge[j] = ti.xe[j] * g[j];
+      gf[j] = ti.xf[j] * g[j];
+    }
   }
 
-  // D: GEMM2, dacc += (s (1 - s))^T (g X_aug)
-  __device__ __forceinline__ void gemm2(const f4 (&dlt)[NT], const f2 (&xb)[4]) {
+  // D: GEMM2, dacc += (s (1 - s))^T (g X_aug): features 0 .. 15 as one 16x16 tile per hidden tile,
+  // features 16 .. D0 + 1 as 4x4 blocks
+  __device__ __forceinline__ void gemm2(const f4 (&dlt)[NT], const float (&ge)[4], const f2 (&gf)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        dacc_e[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(dlt[t][j], ge[j], dacc_e[t], 0, 0, 0);
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        dacc[t][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(dlt[t][j], xb[j][0], dacc[t][0], 0, 0, 0);
-        dacc[t][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(dlt[t][j], xb[j][1], dacc[t][1], 0, 0, 0);
+        dacc_f[t][0] = __builtin_amdgcn_mfma_f32_4x4x1f32(dlt[t][j], gf[j][0], dacc_f[t][0], 0, 0, 0);
+        dacc_f[t][1] = __builtin_amdgcn_mfma_f32_4x4x1f32(dlt[t][j], gf[j][1], dacc_f[t][1], 0, 0, 0);
       }
     }
   }
 
   // Software-pipelined loop over full, aligned tiles [tb, te).  Iteration i issues the loads of tile
   // i + 2, GEMM1 of tile i + 1, the pointwise work of tile i and GEMM2 of tile i - 1, all in one
-  // basic block, so the matrix pipe (42 MFMAs per tile) and the vector ALU (the pointwise work) run
-  // side by side inside one wave.  Lanes whose operand slot is the constant-one feature or padding
-  // read it from a small constant table through a per-lane pointer with stride zero, so no select
-  // sits between a load and its use.
+  // basic block.
   template <int LIK, bool LAST>
   __device__ __forceinline__ void fast_loop(const StepCtx& cx, const ModelConsts& mc, int tb, int te,
                                             int n, int q) {
-    const AugTable<D0>* aug = aug_table<D0>();
-    const size_t tile_floats = (size_t)16 * D0;
-    // A operand: pairs 0 .. KP-2 are always real features; the last pair of lane group q = 3 is
-    // the (1, 0) constant
-    const float* pa = cx.X + (size_t)n * D0 + KS * q;
-    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
-    const float* pa_last0 = a_const ? aug->one : pa + (size_t)tb * tile_floats + 2 * (KP - 1);
-    const unsigned sa_last = a_const ? 0u : (unsigned)tile_floats;
-    // B operand of GEMM2: feature pair 2n, 2n+1 of rows 4q + j
-    const bool b_const = 2 * n >= D0;
-    const float* pb0 = b_const ? (2 * n == D0 ? aug->one : aug->zero)
-                               : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 2 * n;
-    const unsigned sb = b_const ? 0u : (unsigned)tile_floats;
-    const float* py = cx.y + 4 * q;
-
-    auto load = [&](TileIn& ti, int tile) {
-      const float* ra = pa + (size_t)tile * tile_floats;
-#pragma unroll
-      for (int i = 0; i < KP - 1; ++i) ti.xa[i] = *reinterpret_cast<const f2*>(ra + 2 * i);
-      const unsigned rel = (unsigned)(tile - tb);
-      ti.xa[KP - 1] = *reinterpret_cast<const f2*>(pa_last0 + (size_t)rel * sa_last);
-      const float* rb = pb0 + (size_t)rel * sb;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) ti.xb[j] = *reinterpret_cast<const f2*>(rb + j * D0);
-      ti.yv = *reinterpret_cast<const f4*>(py + (size_t)tile * 16);
-    };
-
+    const PlainPtrs pp = plain_ptrs(cx, tb, n, q);
     TileIn t0, t1, t2;  // tiles i, i + 1, i + 2
     f4 acc_cur[NT], acc_nxt[NT], dlt_prev[NT];
-    f2 xb_prev[4];
-    load(t0, tb);
-    load(t1, tb + 1 < te ? tb + 1 : tb);
+    float ge_prev[4];
+    f2 gf_prev[4];
+    load_plain(t0, pp, tb);
+    load_plain(t1, pp, tb + 1 < te ? tb + 1 : tb);
     gemm1(t0.xa, acc_cur);
 #pragma unroll
     for (int t = 0; t < NT; ++t) dlt_prev[t] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) xb_prev[j] = t0.xb[j];
+    for (int j = 0; j < 4; ++j) {
+      ge_prev[j] = 0.0f;
+      gf_prev[j] = f2{0.f, 0.f};
+    }
     for (int i = tb; i < te; ++i) {
-      load(t2, i + 2 < te ? i + 2 : te - 1);
-      gemm1(t1.xa, acc_nxt);                                       // tile i + 1
-      gemm2(dlt_prev, xb_prev);                                    // tile i - 1 (zero delta at i = tb)
-      f2 xg[4];
-      pointwise<LIK, LAST, true>(acc_cur, t0.yv, t0.xb, xg, cx, mc, i * 16, n, q);  // tile i
+      load_plain(t2, pp, i + 2 < te ? i + 2 : te - 1);
+      gemm1(t1.xa, acc_nxt);                  // tile i + 1
+      gemm2(dlt_prev, ge_prev, gf_prev);      // tile i - 1 (zero operands at i = tb)
+      float ge[4];
+      f2 gf[4];
+      pointwise<LIK, LAST, true>(acc_cur, t0, ge, gf, cx, mc, i * 16, n, q);  // tile i
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         dlt_prev[t] = acc_cur[t];
         acc_cur[t] = acc_nxt[t];
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xb_prev[j] = xg[j];
+      for (int j = 0; j < 4; ++j) {
+        ge_prev[j] = ge[j];
+        gf_prev[j] = gf[j];
+      }
       t0 = t1;
       t1 = t2;
     }
-    gemm2(dlt_prev, xb_prev);  // tile te - 1
+    gemm2(dlt_prev, ge_prev, gf_prev);  // tile te - 1
   }
 
-  // Plain loop over full, aligned tiles [tb, te): loads one tile ahead, then GEMM1, pointwise work
-  // and GEMM2 of the current tile back to back.  Needs few registers, so more waves fit a SIMD and
-  // fill each other's dependency and memory stalls.
+  // Plain loop over full, aligned tiles [tb, te): loads two tiles ahead (as far as the compiler
+  // leaves them there), then GEMM1, pointwise work and GEMM2 of the current tile back to back.
   template <int LIK, bool LAST>
   __device__ __forceinline__ void simple_loop(const StepCtx& cx, const ModelConsts& mc, int tb,
                                               int te, int n, int q) {
-    const AugTable<D0>* aug = aug_table<D0>();
-    const size_t tile_floats = (size_t)16 * D0;
-    const float* pa = cx.X + (size_t)n * D0 + KS * q;
-    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
-    const float* pa_last0 = a_const ? aug->one : pa + (size_t)tb * tile_floats + 2 * (KP - 1);
-    const unsigned sa_last = a_const ? 0u : (unsigned)tile_floats;
-    const bool b_const = 2 * n >= D0;
-    const float* pb0 = b_const ? (2 * n == D0 ? aug->one : aug->zero)
-                               : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 2 * n;
-    const unsigned sb = b_const ? 0u : (unsigned)tile_floats;
-    const float* py = cx.y + 4 * q;
-    auto load = [&](TileIn& ti, int tile) {
-      const float* ra = pa + (size_t)tile * tile_floats;
-#pragma unroll
-      for (int i = 0; i < KP - 1; ++i) ti.xa[i] = *reinterpret_cast<const f2*>(ra + 2 * i);
-      const unsigned rel = (unsigned)(tile - tb);
-      ti.xa[KP - 1] = *reinterpret_cast<const f2*>(pa_last0 + (size_t)rel * sa_last);
-      const float* rb = pb0 + (size_t)rel * sb;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) ti.xb[j] = *reinterpret_cast<const f2*>(rb + j * D0);
-      ti.yv = *reinterpret_cast<const f4*>(py + (size_t)tile * 16);
-    };
-    TileIn cur, nx1, nx2;  // loads run two tiles ahead of their use
-    load(cur, tb);
-    load(nx1, tb + 1 < te ? tb + 1 : te - 1);
+    const PlainPtrs pp = plain_ptrs(cx, tb, n, q);
+    TileIn cur, nx1, nx2;
+    load_plain(cur, pp, tb);
+    load_plain(nx1, pp, tb + 1 < te ? tb + 1 : te - 1);
     for (int i = tb; i < te; ++i) {
-      load(nx2, i + 2 < te ? i + 2 : te - 1);
+      load_plain(nx2, pp, i + 2 < te ? i + 2 : te - 1);
       f4 acc[NT];
-      f2 xg[4];
+      float ge[4];
+      f2 gf[4];
       gemm1(cur.xa, acc);
-      pointwise<LIK, LAST, true>(acc, cur.yv, cur.xb, xg, cx, mc, i * 16, n, q);
-      gemm2(acc, xg);
+      pointwise<LIK, LAST, true>(acc, cur, ge, gf, cx, mc, i * 16, n, q);
+      gemm2(acc, ge, gf);
       cur = nx1;
       nx1 = nx2;
     }
@@ -368,21 +399,22 @@ struct MfmaLayer {
   // The compiler sinks ordinary loads of read-only data next to their first use, which undoes any
   // prefetch written in the source.  Here the loads are issued by inline assembly, which it neither
   // moves nor waits for, two tiles ahead of their use into three rotating register sets, and the
-  // waits are explicit: s_waitcnt vmcnt(14) leaves the two newer tiles (7 loads each) in flight.
+  // waits are explicit: s_waitcnt vmcnt(2 * N_LOADS) leaves the two newer tiles in flight.
   // Memory operations the compiler adds on its own (the last step's log-likelihood rows, spills)
   // only make these waits more conservative, never too short: vmcnt counts every outstanding
   // operation in issue order.
+  static constexpr int N_LOADS = 11;
   struct TileRaw {
-    f4 xa01;   // GEMM1 operand, k-pairs 0 and 1
-    f2 xa2;    // k-pair 2 (the (1, 0) constant in lane group q = 3)
-    f2 xb[4];  // GEMM2 operand
-    f4 yv;
+    f4 xa01;  // GEMM1 operand, k-pairs 0 and 1
+    TileIn t; // t.xa[KP - 1]: k-pair 2 (the (1, 0) constant in lane group q = 3); t.xa[0 .. 1] are
+              // filled from xa01 when the tile is used
   };
   template <int N>
-  static __device__ __forceinline__ void wait_tile(TileRaw& t) {
+  static __device__ __forceinline__ void wait_tile(TileRaw& r) {
     asm volatile("s_waitcnt vmcnt(%[cnt])"
-                 : "+v"(t.xa01), "+v"(t.xa2), "+v"(t.xb[0]), "+v"(t.xb[1]), "+v"(t.xb[2]), "+v"(t.xb[3]),
-                   "+v"(t.yv)
+                 : "+v"(r.xa01), "+v"(r.t.xa[KP - 1]), "+v"(r.t.xe[0]), "+v"(r.t.xe[1]), "+v"(r.t.xe[2]),
+                   "+v"(r.t.xe[3]), "+v"(r.t.xf[0]), "+v"(r.t.xf[1]), "+v"(r.t.xf[2]), "+v"(r.t.xf[3]),
+                   "+v"(r.t.y1)
                  : [cnt] "n"(N)
                  : "memory");
   }
@@ -395,23 +427,23 @@ struct MfmaLayer {
     // per-lane offset that never changes: no vector instruction is spent on addresses.  Lanes whose
     // operand slot is the constant-one feature or padding do not load at all: their registers are
     // set once, below, and the loads of those slots run with these lanes masked out of EXEC.
+    const int jj = n & 3;
     const unsigned oa = (unsigned)((n * D0 + KS * q) * 4);
     const unsigned ol = oa + 2 * (KP - 1) * 4;
-    const unsigned ob = (unsigned)(((4 * q) * D0 + 2 * n) * 4);
-    const unsigned oy = (unsigned)(4 * q * 4);
+    const unsigned oe = (unsigned)(((4 * q) * D0 + n) * 4);
+    const unsigned of = (unsigned)(((4 * q) * D0 + 16 + 2 * jj) * 4);
+    const unsigned oy = (unsigned)((4 * q + jj) * 4);
     const bool a_const = KS * q + 2 * (KP - 1) >= D0;
-    const bool b_const = 2 * n >= D0;
+    const bool f_const = 16 + 2 * jj >= D0;
     const unsigned long long mask_a = __builtin_amdgcn_ballot_w64(!a_const);
-    const unsigned long long mask_b = __builtin_amdgcn_ballot_w64(!b_const);
-    const f2 const_a = f2{1.0f, 0.0f};
-    const f2 const_b = f2{2 * n == D0 ? 1.0f : 0.0f, 0.0f};
+    const unsigned long long mask_f = __builtin_amdgcn_ballot_w64(!f_const);
     int nxt = tb;  // tiles are issued in order, one call each; past the last tile the base stays
-    auto issue = [&](TileRaw& t) {  // exactly 7 loads
+    auto issue = [&](TileRaw& r) {  // exactly N_LOADS loads
       const int tile = nxt < te ? nxt : te - 1;
       ++nxt;
       const float* bx = cx.X + (size_t)tile * (16 * D0);
       const float* by = cx.y + (size_t)tile * 16;
-      // One block for the seven loads.  The leading s_nop gives the five wait states a memory
+      // One block for the eleven loads.  The leading s_nop gives the five wait states a memory
       // instruction needs after a VALU instruction wrote one of its SGPR operands (the compiler
       // reloads spilled SGPRs with v_readlane and does not see the loads inside the assembly, so it
       // would not insert them itself).  EXEC is saved on entry and put back.  The pure outputs are
@@ -422,37 +454,44 @@ struct MfmaLayer {
           "s_mov_b64 %[sv], exec\n\t"
           "s_nop 3\n\t"
           "global_load_dwordx4 %[xa01], %[oa], %[bx]\n\t"
+          "global_load_dword %[xe0], %[oe], %[bx]\n\t"
+          "global_load_dword %[xe1], %[oe], %[bx] offset:%[r1]\n\t"
+          "global_load_dword %[xe2], %[oe], %[bx] offset:%[r2]\n\t"
+          "global_load_dword %[xe3], %[oe], %[bx] offset:%[r3]\n\t"
+          "global_load_dword %[y1], %[oy], %[by]\n\t"
           "s_and_b64 exec, %[sv], %[ma]\n\t"
           "global_load_dwordx2 %[xa2], %[ol], %[bx]\n\t"
-          "s_and_b64 exec, %[sv], %[mb]\n\t"
-          "global_load_dwordx2 %[xb0], %[ob], %[bx]\n\t"
-          "global_load_dwordx2 %[xb1], %[ob], %[bx] offset:%[r1]\n\t"
-          "global_load_dwordx2 %[xb2], %[ob], %[bx] offset:%[r2]\n\t"
-          "global_load_dwordx2 %[xb3], %[ob], %[bx] offset:%[r3]\n\t"
-          "s_mov_b64 exec, %[sv]\n\t"
-          "global_load_dwordx4 %[yv], %[oy], %[by]"
-          : [xa01] "=&v"(t.xa01), [xa2] "+v"(t.xa2), [xb0] "+v"(t.xb[0]), [xb1] "+v"(t.xb[1]),
-            [xb2] "+v"(t.xb[2]), [xb3] "+v"(t.xb[3]), [yv] "=&v"(t.yv), [sv] "=&s"(exec_save)
-          : [oa] "v"(oa), [ol] "v"(ol), [ob] "v"(ob), [oy] "v"(oy), [bx] "s"(bx), [by] "s"(by),
-            [ma] "s"(mask_a), [mb] "s"(mask_b), [r1] "n"(D0 * 4), [r2] "n"(2 * D0 * 4),
+          "s_and_b64 exec, %[sv], %[mf]\n\t"
+          "global_load_dwordx2 %[xf0], %[of], %[bx]\n\t"
+          "global_load_dwordx2 %[xf1], %[of], %[bx] offset:%[r1]\n\t"
+          "global_load_dwordx2 %[xf2], %[of], %[bx] offset:%[r2]\n\t"
+          "global_load_dwordx2 %[xf3], %[of], %[bx] offset:%[r3]\n\t"
+          "s_mov_b64 exec, %[sv]"
+          : [xa01] "=&v"(r.xa01), [xa2] "+v"(r.t.xa[KP - 1]), [xe0] "=&v"(r.t.xe[0]), [xe1] "=&v"(r.t.xe[1]),
+            [xe2] "=&v"(r.t.xe[2]), [xe3] "=&v"(r.t.xe[3]), [xf0] "+v"(r.t.xf[0]), [xf1] "+v"(r.t.xf[1]),
+            [xf2] "+v"(r.t.xf[2]), [xf3] "+v"(r.t.xf[3]), [y1] "=&v"(r.t.y1), [sv] "=&s"(exec_save)
+          : [oa] "v"(oa), [ol] "v"(ol), [oe] "v"(oe), [of] "v"(of), [oy] "v"(oy), [bx] "s"(bx), [by] "s"(by),
+            [ma] "s"(mask_a), [mf] "s"(mask_f), [r1] "n"(D0 * 4), [r2] "n"(2 * D0 * 4),
             [r3] "n"(3 * D0 * 4)
           : "memory", "scc");
     };
-    auto preset = [&](TileRaw& t) {
-      t.xa2 = const_a;
+    auto preset = [&](TileRaw& r) {
+      r.t.xa[KP - 1] = f2{1.0f, 0.0f};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) t.xb[j] = const_b;
+      for (int j = 0; j < 4; ++j) r.t.xf[j] = const_f(jj);
     };
-    auto compute = [&](TileRaw& t, int tile) {
-      const f2 xa[KP] = {f2{t.xa01[0], t.xa01[1]}, f2{t.xa01[2], t.xa01[3]}, t.xa2};
+    auto compute = [&](TileRaw& r, int tile) {
+      r.t.xa[0] = f2{r.xa01[0], r.xa01[1]};
+      r.t.xa[1] = f2{r.xa01[2], r.xa01[3]};
       f4 acc[NT];
-      f2 xg[4];
-      gemm1(xa, acc);
-      pointwise<LIK, LAST, true>(acc, t.yv, t.xb, xg, cx, mc, tile * 16, n, q);
+      float ge[4];
+      f2 gf[4];
+      gemm1(r.t.xa, acc);
+      pointwise<LIK, LAST, true>(acc, r.t, ge, gf, cx, mc, tile * 16, n, q);
       // keep the stages apart: left to itself the scheduler may feed each GEMM2 operand to its
       // MFMAs the moment it is computed, which puts two wait states in front of every other MFMA
       __builtin_amdgcn_sched_barrier(0);
-      gemm2(acc, xg);
+      gemm2(acc, ge, gf);
       __builtin_amdgcn_sched_barrier(0);
     };
     TileRaw A, B, C;
@@ -471,13 +510,13 @@ struct MfmaLayer {
     const bool balance = cx.progress != nullptr;
     for (; i + 3 <= te; i += 3) {
       issue(C);
-      wait_tile<14>(A);
+      wait_tile<2 * N_LOADS>(A);
       compute(A, i);
       issue(A);
-      wait_tile<14>(B);
+      wait_tile<2 * N_LOADS>(B);
       compute(B, i + 1);
       issue(B);
-      wait_tile<14>(C);
+      wait_tile<2 * N_LOADS>(C);
       compute(C, i + 2);
       if (balance) {
         // all operands are wave-uniform: the registers live only across these three instructions
@@ -518,11 +557,12 @@ struct MfmaLayer {
     for (int tile = max(tb, fast_end); tile < te; ++tile) {
       TileIn ti;
       f4 acc[NT];
+      float ge[4];
+      f2 gf[4];
       load_tile_safe(ti, cx, tile * 16, n, q);
-      f2 xg[4];
       gemm1(ti.xa, acc);
-      pointwise<LIK, LAST, false>(acc, ti.yv, ti.xb, xg, cx, mc, tile * 16, n, q);
-      gemm2(acc, xg);
+      pointwise<LIK, LAST, false>(acc, ti, ge, gf, cx, mc, tile * 16, n, q);
+      gemm2(acc, ge, gf);
     }
   }
 
@@ -536,18 +576,31 @@ struct MfmaLayer {
     const float gr4 = 4.0f * gr;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
+      // features 0 .. 15: lane (n, q), component i: c = 16 t + 4 q + i, f = n
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int f = 2 * n + u;
+      for (int i = 0; i < 4; ++i) {
+        const int c = 16 * t + 4 * q + i;
+        if (c < D1) slot[n * D1 + c] = dacc_e[t][i] * (gr4 * s_w[oW2 + c]);
+      }
+      // features 16 .. D0 + 1: lane (n, q), component i: c = 16 t + 4 (n >> 2) + i,
+      // f = 16 + 2 (n & 3) + fb, partial of row group q: the four row groups in a fixed order
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int c = 16 * t + 4 * q + j;
-          if (c < D1) {
-            const float v = dacc[t][u][j] * (gr4 * s_w[oW2 + c]);
-            if (f < D0) slot[f * D1 + c] = v;
-            else if (f == D0) slot[oB1 + c] = v;
-          } else if (c == D1 && f == D0) {
-            slot[oB2] = gr4 * dacc[t][u][j];  // sum of g over this wave's rows
+      for (int fb = 0; fb < 2; ++fb) {
+        const int f = 16 + 2 * (n & 3) + fb;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v = dacc_f[t][fb][i];
+          v += __shfl_xor(v, 16);
+          v += __shfl_xor(v, 32);
+          const int c = 16 * t + 4 * (n >> 2) + i;
+          if (q == 0) {
+            if (c < D1) {
+              const float w = v * (gr4 * s_w[oW2 + c]);
+              if (f < D0) slot[f * D1 + c] = w;
+              else if (f == D0) slot[oB1 + c] = w;
+            } else if (c == D1 && f == D0) {
+              slot[oB2] = gr4 * v;  // sum of g over this wave's rows
+            }
           }
         }
       }
