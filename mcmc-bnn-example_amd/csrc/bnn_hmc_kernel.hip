@@ -66,6 +66,7 @@ struct FfmaLayer {
     b2 = s_w[oB2];
   }
 
+  __device__ __forceinline__ void prime(const StepCtx&) {}  // nothing is carried from step to step
   __device__ __forceinline__ void zero_acc() {
 #pragma unroll
     for (int i = 0; i < HU; ++i) {
@@ -165,7 +166,7 @@ struct FfmaLayer {
   }
 
   template <int LIK>
-  __device__ __forceinline__ void write_partials(float* slot, const float*) {
+  __device__ __forceinline__ void write_partials(float* slot, const float*, bool) {
     const int lane = threadIdx.x & 63, cc = lane & 7, rg = lane >> 3;
 #pragma unroll
     for (int i = 0; i < HU; ++i) {
@@ -304,6 +305,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   }
 
   Layer layer;
+  layer.prime(cx);  // the first tiles of the first gradient evaluation
   bool ok = true;
   // optional per-phase cycle accounting (thread 0 of each workgroup)
   unsigned long long ph[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -376,7 +378,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         layer.template run_tiles<LIK, false>(cx, mc);
       }
       BNN_PHASE(2)  // tile loop
-      layer.template write_partials<LIK>(s_slots[wave], s_w);
+      layer.template write_partials<LIK>(s_slots[wave], s_w, last);
       __syncthreads();
       BNN_PHASE(3)  // wave partials -> LDS + sync
       // ---- stage 1: fixed-order sum over this workgroup's waves -> global partial record ----

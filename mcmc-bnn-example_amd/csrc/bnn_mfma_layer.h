@@ -274,8 +274,12 @@ struct MfmaLayer {
       dz = rz * ratio;
       gz = dz * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(dz, dz, mc.df));
     }
-    float g[4] = {row16_bcast<0>(gz), row16_bcast<1>(gz), row16_bcast<2>(gz), row16_bcast<3>(gz)};
+    float g[4];
     if (!FULL) {
+      g[0] = row16_bcast<0>(gz);
+      g[1] = row16_bcast<1>(gz);
+      g[2] = row16_bcast<2>(gz);
+      g[3] = row16_bcast<3>(gz);
 #pragma unroll
       for (int j = 0; j < 4; ++j) g[j] = row0 + 4 * q + j < cx.n ? g[j] : 0.0f;  // mcmc_step_ffma.h:301
     }
@@ -294,20 +298,82 @@ struct MfmaLayer {
         }
       }
     }
+    if (FULL) {
+      // every consumer of g takes it straight out of its bank of gz (a DPP operand), so the four
+      // values are never copied into registers of their own
+      consume_g(acc, gz, ti, ge, gf);
+    } else {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dw2s[t] = __builtin_fmaf(g[j], acc[t][j], dw2s[t]);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        ge[j] = ti.xe[j] * g[j];
+        gf[j] = ti.xf[j] * g[j];
+      }
+    }
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float sg = acc[t][j];
-        dw2s[t] = __builtin_fmaf(g[j], sg, dw2s[t]);
         acc[t][j] = __builtin_fmaf(-sg, sg, sg);
       }
     }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      ge[j] = ti.xe[j] * g[j];
-      gf[j] = ti.xf[j] * g[j];
-    }
+  }
+
+  // dw2s[t] += g_j s[t][j] and (ge, gf)[j] = g_j (xe, xf)[j], where g_j sits in bank j of gz and is
+  // read through a DPP row broadcast (no builtin pairs a broadcast with a multiply-add, hence the
+  // assembly; the leading s_nop keeps the DPP reads two wait states behind the instruction that
+  // wrote gz).  The order of the additions into dw2s[t] is j = 0, 1, 2, 3.
+  __device__ __forceinline__ void consume_g(const f4 (&s)[NT], float gz, const TileIn& ti, float (&ge)[4],
+                                            f2 (&gf)[4]) {
+    static_assert(NT == 3, "operand lists are written for three hidden tiles");
+#define BNN_BC(j) " row_newbcast:" #j " row_mask:0xf bank_mask:0xf\n\t"
+    asm("s_nop 1\n\t"
+        "v_fmac_f32_dpp %[d0], %[g], %[s00]" BNN_BC(0)
+        "v_fmac_f32_dpp %[d1], %[g], %[s10]" BNN_BC(0)
+        "v_fmac_f32_dpp %[d2], %[g], %[s20]" BNN_BC(0)
+        "v_fmac_f32_dpp %[d0], %[g], %[s01]" BNN_BC(4)
+        "v_fmac_f32_dpp %[d1], %[g], %[s11]" BNN_BC(4)
+        "v_fmac_f32_dpp %[d2], %[g], %[s21]" BNN_BC(4)
+        "v_fmac_f32_dpp %[d0], %[g], %[s02]" BNN_BC(8)
+        "v_fmac_f32_dpp %[d1], %[g], %[s12]" BNN_BC(8)
+        "v_fmac_f32_dpp %[d2], %[g], %[s22]" BNN_BC(8)
+        "v_fmac_f32_dpp %[d0], %[g], %[s03]" BNN_BC(12)
+        "v_fmac_f32_dpp %[d1], %[g], %[s13]" BNN_BC(12)
+        "v_fmac_f32_dpp %[d2], %[g], %[s23] row_newbcast:12 row_mask:0xf bank_mask:0xf"
+        : [d0] "+v"(dw2s[0]), [d1] "+v"(dw2s[1]), [d2] "+v"(dw2s[2])
+        : [g] "v"(gz), [s00] "v"(s[0][0]), [s01] "v"(s[0][1]), [s02] "v"(s[0][2]), [s03] "v"(s[0][3]),
+          [s10] "v"(s[1][0]), [s11] "v"(s[1][1]), [s12] "v"(s[1][2]), [s13] "v"(s[1][3]),
+          [s20] "v"(s[2][0]), [s21] "v"(s[2][1]), [s22] "v"(s[2][2]), [s23] "v"(s[2][3]));
+    float f00, f01, f10, f11, f20, f21, f30, f31;
+    asm("s_nop 1\n\t"
+        "v_mul_f32_dpp %[e0], %[g], %[x0]" BNN_BC(0)
+        "v_mul_f32_dpp %[a0], %[g], %[p0]" BNN_BC(0)
+        "v_mul_f32_dpp %[b0], %[g], %[r0]" BNN_BC(0)
+        "v_mul_f32_dpp %[e1], %[g], %[x1]" BNN_BC(4)
+        "v_mul_f32_dpp %[a1], %[g], %[p1]" BNN_BC(4)
+        "v_mul_f32_dpp %[b1], %[g], %[r1]" BNN_BC(4)
+        "v_mul_f32_dpp %[e2], %[g], %[x2]" BNN_BC(8)
+        "v_mul_f32_dpp %[a2], %[g], %[p2]" BNN_BC(8)
+        "v_mul_f32_dpp %[b2], %[g], %[r2]" BNN_BC(8)
+        "v_mul_f32_dpp %[e3], %[g], %[x3]" BNN_BC(12)
+        "v_mul_f32_dpp %[a3], %[g], %[p3]" BNN_BC(12)
+        "v_mul_f32_dpp %[b3], %[g], %[r3] row_newbcast:12 row_mask:0xf bank_mask:0xf"
+        : [e0] "=&v"(ge[0]), [e1] "=&v"(ge[1]), [e2] "=&v"(ge[2]), [e3] "=&v"(ge[3]), [a0] "=&v"(f00),
+          [b0] "=&v"(f01), [a1] "=&v"(f10), [b1] "=&v"(f11), [a2] "=&v"(f20), [b2] "=&v"(f21),
+          [a3] "=&v"(f30), [b3] "=&v"(f31)
+        : [g] "v"(gz), [x0] "v"(ti.xe[0]), [x1] "v"(ti.xe[1]), [x2] "v"(ti.xe[2]), [x3] "v"(ti.xe[3]),
+          [p0] "v"(ti.xf[0][0]), [r0] "v"(ti.xf[0][1]), [p1] "v"(ti.xf[1][0]), [r1] "v"(ti.xf[1][1]),
+          [p2] "v"(ti.xf[2][0]), [r2] "v"(ti.xf[2][1]), [p3] "v"(ti.xf[3][0]), [r3] "v"(ti.xf[3][1]));
+#undef BNN_BC
+    gf[0] = f2{f00, f01};
+    gf[1] = f2{f10, f11};
+    gf[2] = f2{f20, f21};
+    gf[3] = f2{f30, f31};
   }
 
   // D: GEMM2, dacc += (s (1 - s))^T (g X_aug): features 0 .. 15 as one 16x16 tile per hidden tile,
@@ -419,66 +485,108 @@ struct MfmaLayer {
                  : "memory");
   }
 
+  // Every load is  base (wave-uniform, in SGPRs, advanced by scalar instructions)  +  a 32-bit
+  // per-lane offset that never changes: no vector instruction is spent on addresses.  Lanes whose
+  // operand slot is the constant-one feature or padding do not load at all: their registers are
+  // set once (preset) and the loads of those slots run with these lanes masked out of EXEC.
+  struct LoadPlan {
+    unsigned oa, ol, oe, of, oy;
+    unsigned long long mask_a, mask_f;
+    int jj;
+  };
+  static __device__ __forceinline__ LoadPlan load_plan(int n, int q) {
+    LoadPlan lp;
+    lp.jj = n & 3;
+    lp.oa = (unsigned)((n * D0 + KS * q) * 4);
+    lp.ol = lp.oa + 2 * (KP - 1) * 4;
+    lp.oe = (unsigned)(((4 * q) * D0 + n) * 4);
+    lp.of = (unsigned)(((4 * q) * D0 + 16 + 2 * lp.jj) * 4);
+    lp.oy = (unsigned)((4 * q + lp.jj) * 4);
+    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
+    const bool f_const = 16 + 2 * lp.jj >= D0;
+    lp.mask_a = __builtin_amdgcn_ballot_w64(!a_const);
+    lp.mask_f = __builtin_amdgcn_ballot_w64(!f_const);
+    return lp;
+  }
+  static __device__ __forceinline__ void preset(TileRaw& r, int jj) {
+    r.t.xa[KP - 1] = f2{1.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r.t.xf[j] = const_f(jj);
+  }
+  // exactly N_LOADS loads of one full tile
+  static __device__ __forceinline__ void issue_tile(TileRaw& r, const StepCtx& cx, const LoadPlan& lp, int tile) {
+    const float* bx = cx.X + (size_t)tile * (16 * D0);
+    const float* by = cx.y + (size_t)tile * 16;
+    // One block for the eleven loads.  The leading s_nop gives the five wait states a memory
+    // instruction needs after a VALU instruction wrote one of its SGPR operands (the compiler
+    // reloads spilled SGPRs with v_readlane and does not see the loads inside the assembly, so it
+    // would not insert them itself).  EXEC is saved on entry and put back.  The pure outputs are
+    // early-clobber: a returning load must not land in a register that still holds an offset of a
+    // load not yet issued.
+    unsigned long long exec_save;
+    asm volatile(
+        "s_mov_b64 %[sv], exec\n\t"
+        "s_nop 3\n\t"
+        "global_load_dwordx4 %[xa01], %[oa], %[bx]\n\t"
+        "global_load_dword %[xe0], %[oe], %[bx]\n\t"
+        "global_load_dword %[xe1], %[oe], %[bx] offset:%[r1]\n\t"
+        "global_load_dword %[xe2], %[oe], %[bx] offset:%[r2]\n\t"
+        "global_load_dword %[xe3], %[oe], %[bx] offset:%[r3]\n\t"
+        "global_load_dword %[y1], %[oy], %[by]\n\t"
+        "s_and_b64 exec, %[sv], %[ma]\n\t"
+        "global_load_dwordx2 %[xa2], %[ol], %[bx]\n\t"
+        "s_and_b64 exec, %[sv], %[mf]\n\t"
+        "global_load_dwordx2 %[xf0], %[of], %[bx]\n\t"
+        "global_load_dwordx2 %[xf1], %[of], %[bx] offset:%[r1]\n\t"
+        "global_load_dwordx2 %[xf2], %[of], %[bx] offset:%[r2]\n\t"
+        "global_load_dwordx2 %[xf3], %[of], %[bx] offset:%[r3]\n\t"
+        "s_mov_b64 exec, %[sv]"
+        : [xa01] "=&v"(r.xa01), [xa2] "+v"(r.t.xa[KP - 1]), [xe0] "=&v"(r.t.xe[0]), [xe1] "=&v"(r.t.xe[1]),
+          [xe2] "=&v"(r.t.xe[2]), [xe3] "=&v"(r.t.xe[3]), [xf0] "+v"(r.t.xf[0]), [xf1] "+v"(r.t.xf[1]),
+          [xf2] "+v"(r.t.xf[2]), [xf3] "+v"(r.t.xf[3]), [y1] "=&v"(r.t.y1), [sv] "=&s"(exec_save)
+        : [oa] "v"(lp.oa), [ol] "v"(lp.ol), [oe] "v"(lp.oe), [of] "v"(lp.of), [oy] "v"(lp.oy), [bx] "s"(bx),
+          [by] "s"(by), [ma] "s"(lp.mask_a), [mf] "s"(lp.mask_f), [r1] "n"(D0 * 4), [r2] "n"(2 * D0 * 4),
+          [r3] "n"(3 * D0 * 4)
+        : "memory", "scc");
+  }
+
+  // the tiles of the fast loop: full, aligned tiles [tile_begin, fast_end)
+  static __device__ __forceinline__ int fast_end_of(const StepCtx& cx) {
+    int fast_end = cx.tile_begin;
+    if (cx.x_vec_ok && cx.y_vec_ok) fast_end = min(cx.tile_end, cx.n / 16);
+    return fast_end;
+  }
+
+  // The data does not change from one gradient evaluation to the next, only the weights do: a wave
+  // goes round its tiles in a circle, and the loop of one evaluation ends with the first two tiles of
+  // the next already in registers (pa, pb), fetched while its own last tiles were being computed, so
+  // that no evaluation starts by waiting for memory.  prime() fetches them for the first evaluation.
+  TileRaw pa, pb;
+  __device__ __forceinline__ void prime(const StepCtx& cx) {
+    if (PIPE != 2) return;
+    const int tb = cx.tile_begin, te = fast_end_of(cx);
+    if (te <= tb) return;
+    const int lane = opaque_tid() & 63;
+    const LoadPlan lp = load_plan(lane & 15, lane >> 4);
+    preset(pa, lp.jj);
+    preset(pb, lp.jj);
+    issue_tile(pa, cx, lp, tb);
+    issue_tile(pb, cx, lp, tb + 1 < te ? tb + 1 : tb);
+    wait_tile<0>(pa);
+    wait_tile<0>(pb);
+  }
+
   template <int LIK, bool LAST>
   __device__ __forceinline__ void prefetch_loop(const StepCtx& cx, const ModelConsts& mc, int tb,
                                                 int te, int n, int q) {
     static_assert(KP == 3, "register sets are laid out for three k-pairs");
-    // Every load is  base (wave-uniform, in SGPRs, advanced by scalar instructions)  +  a 32-bit
-    // per-lane offset that never changes: no vector instruction is spent on addresses.  Lanes whose
-    // operand slot is the constant-one feature or padding do not load at all: their registers are
-    // set once, below, and the loads of those slots run with these lanes masked out of EXEC.
-    const int jj = n & 3;
-    const unsigned oa = (unsigned)((n * D0 + KS * q) * 4);
-    const unsigned ol = oa + 2 * (KP - 1) * 4;
-    const unsigned oe = (unsigned)(((4 * q) * D0 + n) * 4);
-    const unsigned of = (unsigned)(((4 * q) * D0 + 16 + 2 * jj) * 4);
-    const unsigned oy = (unsigned)((4 * q + jj) * 4);
-    const bool a_const = KS * q + 2 * (KP - 1) >= D0;
-    const bool f_const = 16 + 2 * jj >= D0;
-    const unsigned long long mask_a = __builtin_amdgcn_ballot_w64(!a_const);
-    const unsigned long long mask_f = __builtin_amdgcn_ballot_w64(!f_const);
-    int nxt = tb;  // tiles are issued in order, one call each; past the last tile the base stays
-    auto issue = [&](TileRaw& r) {  // exactly N_LOADS loads
-      const int tile = nxt < te ? nxt : te - 1;
-      ++nxt;
-      const float* bx = cx.X + (size_t)tile * (16 * D0);
-      const float* by = cx.y + (size_t)tile * 16;
-      // One block for the eleven loads.  The leading s_nop gives the five wait states a memory
-      // instruction needs after a VALU instruction wrote one of its SGPR operands (the compiler
-      // reloads spilled SGPRs with v_readlane and does not see the loads inside the assembly, so it
-      // would not insert them itself).  EXEC is saved on entry and put back.  The pure outputs are
-      // early-clobber: a returning load must not land in a register that still holds an offset of a
-      // load not yet issued.
-      unsigned long long exec_save;
-      asm volatile(
-          "s_mov_b64 %[sv], exec\n\t"
-          "s_nop 3\n\t"
-          "global_load_dwordx4 %[xa01], %[oa], %[bx]\n\t"
-          "global_load_dword %[xe0], %[oe], %[bx]\n\t"
-          "global_load_dword %[xe1], %[oe], %[bx] offset:%[r1]\n\t"
-          "global_load_dword %[xe2], %[oe], %[bx] offset:%[r2]\n\t"
-          "global_load_dword %[xe3], %[oe], %[bx] offset:%[r3]\n\t"
-          "global_load_dword %[y1], %[oy], %[by]\n\t"
-          "s_and_b64 exec, %[sv], %[ma]\n\t"
-          "global_load_dwordx2 %[xa2], %[ol], %[bx]\n\t"
-          "s_and_b64 exec, %[sv], %[mf]\n\t"
-          "global_load_dwordx2 %[xf0], %[of], %[bx]\n\t"
-          "global_load_dwordx2 %[xf1], %[of], %[bx] offset:%[r1]\n\t"
-          "global_load_dwordx2 %[xf2], %[of], %[bx] offset:%[r2]\n\t"
-          "global_load_dwordx2 %[xf3], %[of], %[bx] offset:%[r3]\n\t"
-          "s_mov_b64 exec, %[sv]"
-          : [xa01] "=&v"(r.xa01), [xa2] "+v"(r.t.xa[KP - 1]), [xe0] "=&v"(r.t.xe[0]), [xe1] "=&v"(r.t.xe[1]),
-            [xe2] "=&v"(r.t.xe[2]), [xe3] "=&v"(r.t.xe[3]), [xf0] "+v"(r.t.xf[0]), [xf1] "+v"(r.t.xf[1]),
-            [xf2] "+v"(r.t.xf[2]), [xf3] "+v"(r.t.xf[3]), [y1] "=&v"(r.t.y1), [sv] "=&s"(exec_save)
-          : [oa] "v"(oa), [ol] "v"(ol), [oe] "v"(oe), [of] "v"(of), [oy] "v"(oy), [bx] "s"(bx), [by] "s"(by),
-            [ma] "s"(mask_a), [mf] "s"(mask_f), [r1] "n"(D0 * 4), [r2] "n"(2 * D0 * 4),
-            [r3] "n"(3 * D0 * 4)
-          : "memory", "scc");
-    };
-    auto preset = [&](TileRaw& r) {
-      r.t.xa[KP - 1] = f2{1.0f, 0.0f};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) r.t.xf[j] = const_f(jj);
+    const LoadPlan lp = load_plan(n, q);
+    // tiles are issued in order, one call each, and after the last tile comes the first again; on
+    // entry pa and pb hold tiles tb and tb + 1 (tb again if there is only one)
+    int nxt = te - tb > 2 ? tb + 2 : tb;
+    auto issue = [&](TileRaw& r) {
+      issue_tile(r, cx, lp, nxt);
+      nxt = nxt + 1 == te ? tb : nxt + 1;
     };
     auto compute = [&](TileRaw& r, int tile) {
       r.t.xa[0] = f2{r.xa01[0], r.xa01[1]};
@@ -494,20 +602,33 @@ struct MfmaLayer {
       gemm2(acc, ge, gf);
       __builtin_amdgcn_sched_barrier(0);
     };
-    TileRaw A, B, C;
-    preset(A);
-    preset(B);
-    preset(C);
-    issue(A);
-    issue(B);
+    TileRaw& A = pa;
+    TileRaw& B = pb;
+    TileRaw C;
+    preset(C, lp.jj);
     // steady state: three tiles per trip, every issue and every wait unconditional.
     // Two waves share a SIMD, and the matrix and vector instructions of both go through one FP32
     // pipe: it stays busy only while both waves have work (each fills the dependency stalls of the
     // other).  The hardware favours the older wave, which would finish its tiles long before the
     // younger one and leave it to run alone, stalls exposed.  So every trip a wave publishes its
-    // tile count in LDS, reads its partner's, and takes the higher priority while it is behind.
+    // tile count in LDS, reads its partner's, and takes the higher priority while it is behind
+    // (once per trip of three tiles: checked after every tile the kernel was 3 % slower).
     int i = tb;
     const bool balance = cx.progress != nullptr;
+    auto keep_pace = [&](int done) {
+      if (balance) {
+        // all operands are wave-uniform: the registers live only across these three instructions
+        const unsigned my_slot = (unsigned)(size_t)(cx.progress + cx.wave);  // LDS byte addresses
+        const unsigned other_slot = (unsigned)(size_t)(cx.progress + cx.partner);
+        int other;
+        asm volatile("ds_write_b32 %1, %2\n\tds_read_b32 %0, %3\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(other)
+                     : "v"(my_slot), "v"(done), "v"(other_slot)
+                     : "memory");
+        if (__builtin_amdgcn_readfirstlane(other) > done) __builtin_amdgcn_s_setprio(2);
+        else __builtin_amdgcn_s_setprio(0);
+      }
+    };
     for (; i + 3 <= te; i += 3) {
       issue(C);
       wait_tile<2 * N_LOADS>(A);
@@ -518,36 +639,42 @@ struct MfmaLayer {
       issue(B);
       wait_tile<2 * N_LOADS>(C);
       compute(C, i + 2);
-      if (balance) {
-        // all operands are wave-uniform: the registers live only across these three instructions
-        const unsigned my_slot = (unsigned)(size_t)(cx.progress + cx.wave);  // LDS byte addresses
-        const unsigned other_slot = (unsigned)(size_t)(cx.progress + cx.partner);
-        const int done = i + 3 - tb;
-        int other;
-        asm volatile("ds_write_b32 %1, %2\n\tds_read_b32 %0, %3\n\ts_waitcnt lgkmcnt(0)"
-                     : "=&v"(other)
-                     : "v"(my_slot), "v"(done), "v"(other_slot)
-                     : "memory");
-        if (__builtin_amdgcn_readfirstlane(other) > done) __builtin_amdgcn_s_setprio(2);
-        else __builtin_amdgcn_s_setprio(0);
-      }
+      keep_pace(i + 3 - tb);
     }
     if (balance) __builtin_amdgcn_s_setprio(0);
+    // the one or two tiles left over sit in A and B (issued at the end of the last trip); the
+    // loads issued from here on are the first tiles of the next evaluation
+    const int left = te - i;
+    if (left >= 1) {
+      issue(C);
+      wait_tile<2 * N_LOADS>(A);
+      compute(A, i);
+    }
+    if (left == 2) {
+      issue(A);
+      wait_tile<2 * N_LOADS>(B);
+      compute(B, i + 1);
+    }
     // no register of a set may be used or reused before its last load has landed
     wait_tile<0>(A);
     wait_tile<0>(B);
     wait_tile<0>(C);
-    // the one or two tiles left over: A and B hold them (issued at the end of the last trip)
-    if (i < te) compute(A, i);
-    if (i + 1 < te) compute(B, i + 1);
+    // tiles tb and tb + 1 back into (pa, pb)
+    if (left == 1) {
+      A = B;
+      B = C;
+    } else if (left == 2) {
+      const TileRaw first = C;
+      B = A;
+      A = first;
+    }
   }
 
   template <int LIK, bool LAST>
   __device__ __forceinline__ void run_tiles(const StepCtx& cx, const ModelConsts& mc) {
     const int lane = opaque_tid() & 63, n = lane & 15, q = lane >> 4;
     const int tb = cx.tile_begin, te = cx.tile_end;
-    int fast_end = tb;
-    if (cx.x_vec_ok && cx.y_vec_ok) fast_end = min(te, cx.n / 16);
+    const int fast_end = fast_end_of(cx);
     if (fast_end > tb) {
       if (PIPE == 1) fast_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
       else if (PIPE == 2) prefetch_loop<LIK, LAST>(cx, mc, tb, fast_end, n, q);
@@ -566,61 +693,106 @@ struct MfmaLayer {
     }
   }
 
+  // a (lower half) + a (upper half) in lanes 0 .. 31 and the same of b in lanes 32 .. 63; one lane
+  // swap and one addition, no trip through LDS.  Written in assembly because the compiler's builtin
+  // for the swap hands back its two results in one register at -O3.  The s_nop is the two wait states
+  // the swap needs after a vector instruction wrote one of its operands; the operands must come from
+  // ordinary vector instructions (not straight from an MFMA, whose longer hazard the compiler cannot
+  // see through the assembly).
+  static __device__ __forceinline__ float fold32(float a, float b) {
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return a + b;
+  }
+  // rows of 16 lanes: (a row 0 + a row 1, b row 0 + b row 1, a row 2 + a row 3, b row 2 + b row 3)
+  static __device__ __forceinline__ float fold16(float a, float b) {
+    asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return a + b;
+  }
+
   // this wave's partial sums -> its LDS slot, indexed by canonical parameter number; the factors
-  // 4 w2[c] left out of the GEMM2 operand and k / k2 left out of g are applied here
+  // 4 w2[c] left out of the GEMM2 operand and k / k2 left out of g are applied here.  `last`: the
+  // log-likelihood difference of the step is written too.
   template <int LIK>
-  __device__ __forceinline__ void write_partials(float* slot, const float* s_w) {
+  __device__ __forceinline__ void write_partials(float* slot, const float* s_w, bool last) {
     const int lane = opaque_tid() & 63, n = lane & 15, q = lane >> 4;
     static_assert(D1 % 16 != 0, "db2 rides in the first padded hidden unit");
+    static_assert(NT == 3, "the row-group sums below are laid out for three hidden tiles");
     const float gr = LIK == 1 ? ratio : 1.0f;
     const float gr4 = 4.0f * gr;
+    // The accumulators of features 16 .. D0 + 1 and of dw2 hold one partial per row group q (the four
+    // rows of 16 lanes); two folds add the four partials of four registers at once and leave each row
+    // of lanes with the total of one of them.  After
+    //     fold16(fold32(x0, y0), fold32(x1, y1))
+    // row q holds the total of (q & 1 ? x1 : x0) for q < 2 and of (q & 1 ? y1 : y0) for q >= 2,
+    // added as (q0 + q2) + (q1 + q3).
+    // ---- factors first, so that the LDS reads are all in flight together ----
+    float fe[NT][4], ff[NT][4];
+    const int cb = 4 * (n >> 2) + (q & 1);  // features 16 ..: hidden unit of this lane after the folds
+    const int f = 16 + 2 * (n & 3) + (q >> 1);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      // features 0 .. 15: lane (n, q), component i: c = 16 t + 4 q + i, f = n
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ce = 16 * t + 4 * q + i, cf = 16 * t + 4 * (n >> 2) + i;
+        fe[t][i] = s_w[oW2 + min(ce, D1 - 1)];
+        ff[t][i] = s_w[oW2 + min(cf, D1 - 1)];
+      }
+    }
+    // ---- features 0 .. 15: lane (n, q), component i: c = 16 t + 4 q + i, f = n ----
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int c = 16 * t + 4 * q + i;
-        if (c < D1) slot[n * D1 + c] = dacc_e[t][i] * (gr4 * s_w[oW2 + c]);
+        if (c < D1) slot[n * D1 + c] = dacc_e[t][i] * (gr4 * fe[t][i]);
       }
-      // features 16 .. D0 + 1: lane (n, q), component i: c = 16 t + 4 (n >> 2) + i,
-      // f = 16 + 2 (n & 3) + fb, partial of row group q: the four row groups in a fixed order
+    }
+    // ---- features 16 .. D0 + 1: before the folds lane (n, q), component i holds
+    //      c = 16 t + 4 (n >> 2) + i, f = 16 + 2 (n & 3) + fb for row group q; after them the lane
+    //      holds c = 16 t + cb + 2 h and the f above.  f = D0 is the bias; the sum of g over the wave's
+    //      rows (db2) has gathered in the first padded hidden unit ----
+    const int fbase = f < D0 ? f * D1 : oB1;
 #pragma unroll
-      for (int fb = 0; fb < 2; ++fb) {
-        const int f = 16 + 2 * (n & 3) + fb;
+    for (int t = 0; t < NT; ++t) {
+      float vs[2][4];  // scaled before the folds: the factor depends on (n, i) only
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float v = dacc_f[t][fb][i];
-          v += __shfl_xor(v, 16);
-          v += __shfl_xor(v, 32);
-          const int c = 16 * t + 4 * (n >> 2) + i;
-          if (q == 0) {
-            if (c < D1) {
-              const float w = v * (gr4 * s_w[oW2 + c]);
-              if (f < D0) slot[f * D1 + c] = w;
-              else if (f == D0) slot[oB1 + c] = w;
-            } else if (c == D1 && f == D0) {
-              slot[oB2] = gr4 * v;  // sum of g over this wave's rows
-            }
-          }
+      for (int i = 0; i < 4; ++i) {
+        const int cf = 16 * t + 4 * (n >> 2) + i;
+        const float fac = gr4 * (cf < D1 ? ff[t][i] : 1.0f);
+        vs[0][i] = dacc_f[t][0][i] * fac;
+        vs[1][i] = dacc_f[t][1][i] * fac;
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const float v = fold16(fold32(vs[0][2 * h], vs[1][2 * h]), fold32(vs[0][2 * h + 1], vs[1][2 * h + 1]));
+        const int c = 16 * t + cb + 2 * h;
+        if (f <= D0) {
+          if (c < D1) slot[fbase + c] = v;
+          else if (c == D1 && f == D0) slot[oB2] = v;
         }
       }
-      // dw2 = sum_rows g h = 2 (sum_rows g s - sum_rows g / 2); the second sum is what the first padded
-      // hidden unit (lane n = D1 % 16 of the last hidden tile, s = 1/2) has accumulated; the four row
-      // groups q in a fixed order
-      const float half_gsum = dpp_move<0x150 + D1 % 16>(dw2s[NT - 1]);  // row_newbcast
-      float v = 2.0f * (dw2s[t] - half_gsum) * gr;
-      v += __shfl_xor(v, 16);
-      v += __shfl_xor(v, 32);
-      const int c = 16 * t + n;
-      if (q == 0 && c < D1) slot[oW2 + c] = v;
     }
-    double d = dl;  // held by lanes n == 0
-    d += shfl_xor_d(d, 16);
-    d += shfl_xor_d(d, 32);
-    if (lane == 0) {
-      const uint64_t bits = double_to_bits(d);
-      slot[P_AL] = __builtin_bit_cast(float, (uint32_t)bits);
-      slot[P_AL + 1] = __builtin_bit_cast(float, (uint32_t)(bits >> 32));
+    // ---- dw2 = sum_rows g h = 2 (sum_rows g s - sum_rows g / 2); the second sum is what the first
+    //      padded hidden unit (lane n = D1 % 16 of the last hidden tile, s = 1/2) has accumulated ----
+    {
+      const float half_gsum = dpp_move<0x150 + D1 % 16>(dw2s[NT - 1]);  // row_newbcast
+      const float v0 = 2.0f * (dw2s[0] - half_gsum) * gr;
+      const float v1 = 2.0f * (dw2s[1] - half_gsum) * gr;
+      const float v2 = 2.0f * (dw2s[2] - half_gsum) * gr;
+      const float v = fold16(fold32(v0, v1), fold32(v2, v2));  // rows: tile 0, tile 2, tile 1, tile 2
+      const int t = q == 0 ? 0 : (q == 2 ? 1 : 2);
+      const int c = 16 * t + n;
+      if (q < 3 && c < D1) slot[oW2 + c] = v;
+    }
+    if (last) {
+      double d = dl;  // held by lanes n == 0
+      d += shfl_xor_d(d, 16);
+      d += shfl_xor_d(d, 32);
+      if (lane == 0) {
+        const uint64_t bits = double_to_bits(d);
+        slot[P_AL] = __builtin_bit_cast(float, (uint32_t)bits);
+        slot[P_AL + 1] = __builtin_bit_cast(float, (uint32_t)(bits >> 32));
+      }
     }
   }
 };

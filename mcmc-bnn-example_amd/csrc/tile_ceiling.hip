@@ -1,6 +1,6 @@
 // Ceiling of the tile loop of the 22 -> 40 -> 1 MFMA trajectory kernel on gfx950: the tile's own
-// instruction mix -- GEMM1 (18 MFMAs 16x16x4), the pointwise stage, GEMM2 (12 MFMAs 16x16x4 + 24 MFMAs 4x4x1), taken from the very
-// header the kernel is built from -- run on registers, with no memory traffic, no barrier and no
+// instruction mix -- GEMM1 (18 MFMAs 16x16x4), the pointwise stage, GEMM2 (12 MFMAs 16x16x4 and
+// 24 MFMAs 4x4x1), taken from the very header the kernel is built from -- run on registers, with no memory traffic, no barrier and no
 // reduction, two waves per SIMD as in the kernel.  FP32 MFMA and vector instructions share one pipe
 // on this chip, so the time per tile is what that instruction mix costs on it; the production loop can
 // come close to this number but not beat it.  Also times the two halves of the mix alone.
@@ -17,7 +17,7 @@
 using namespace bnn;
 using Layer = MfmaLayer<22, 40, 2>;
 
-// MODE 0: the whole tile; 1: the 42 MFMAs alone; 2: the pointwise stage alone
+// MODE 0: the whole tile; 1: the MFMAs alone; 2: the pointwise stage alone
 template <int MODE>
 __global__ __launch_bounds__(512) void tile_kernel(float* out, unsigned long long* cycles, int tiles,
                                                    ModelConsts mc, const float* w) {
@@ -118,10 +118,12 @@ int run(const char* what, int tiles, float* d_out, unsigned long long* d_cyc, co
     mean += (double)cyc[2 * i] / wgs;
     real += (double)cyc[2 * i + 1] / wgs;
   }
-  // two waves per SIMD run side by side for the whole launch: a SIMD does 2 * tiles tiles in `mean` cycles
-  std::printf("%-34s %9.3f ms (events) %9.3f ms (100 MHz counter) %12.0f shader-clock ticks per wave = %.0f MHz, "
-              "%8.1f ticks per tile and SIMD\n",
-              what, ms, real * 1e-5, mean, mean / (real * 1e-2), mean / (2.0 * tiles));
+  // A SIMD holds two waves and issues the older one first, so a wave's own start-to-end ticks say little;
+  // the launch as a whole takes 2 * tiles tiles per SIMD, and the shader clock is the ratio of the two
+  // counters that one wave read.
+  const double mhz = mean / (real * 1e-2);
+  std::printf("%-34s %9.3f ms (events), shader clock %.0f MHz, %8.1f cycles per tile and SIMD\n", what, ms, mhz,
+              ms * 1e-3 * mhz * 1e6 / (2.0 * tiles));
   return 0;
 }
 
