@@ -62,45 +62,107 @@ def test_first_50_transitions_at_full_size(config0_chain, orc):
     assert 5e-6 < c["state"]["eps"] < 1e-4
 
 
+def _log_alpha_f64(orc, X, y, w0, eps, t):
+    """One transition of configs[0] in float64, written out in numpy from the model's definition
+    (tanh hidden layer, Gaussian likelihood sigma = 0.01, prior N(0, 0.1^2), leapfrog with half kicks
+    at both ends, main.h:207-265): the value both FP32 implementations approximate.  Only the start
+    momentum is taken from the oracle (its RNG is pinned bit for bit elsewhere)."""
+    X64, y64 = X.astype(np.float64).reshape(N_FULL, D0), y.astype(np.float64)
+    sig, sp = 0.01, 0.1
+
+    def logpost_and_grad(w):
+        W1 = w[:D0 * D1].reshape(D0, D1)
+        b1 = w[D0 * D1:D0 * D1 + D1]
+        W2 = w[D0 * D1 + D1:D0 * D1 + 2 * D1]
+        H = np.tanh(X64 @ W1 + b1)
+        r = (y64 - (H @ W2 + w[-1])) / sig
+        lp = -0.5 * np.sum(r * r) - 0.5 * np.sum((w / sp) ** 2)
+        d = r / sig
+        dH = np.outer(d, W2) * (1.0 - H * H)
+        g = np.concatenate([(X64.T @ dH).ravel(), dH.sum(0), H.T @ d, [d.sum()]]) - w / sp ** 2
+        return lp, g
+
+    m = orc.momentum(0, 0, t, P).astype(np.float64)
+    w, eps = np.asarray(w0, dtype=np.float64), float(eps)
+    lp0, g = logpost_and_grad(w)
+    k0 = 0.5 * np.sum(m * m)
+    for step in range(L_FULL):
+        m = m + (0.5 * eps if step == 0 else eps) * g
+        w = w + eps * m
+        lp1, g = logpost_and_grad(w)
+    m = m + 0.5 * eps * g
+    return (lp1 - lp0) + (k0 - 0.5 * np.sum(m * m))
+
+
+def _rms(d):
+    d = np.asarray(d, dtype=np.float64)
+    return float(np.sqrt(np.mean(d * d)))
+
+
 def test_20_transitions_from_the_adapted_state_at_full_size(config0_chain, orc):
     """The second leg: from the state the burn-in ends in (step size about 2e-5, weights of order
-    10), 20 transitions of 1000 leapfrog steps on the GPU and on the oracle, same RNG counters.
+    10), 20 transitions of 1000 leapfrog steps.  Each one is run on the GPU and, from the very state
+    the GPU started it in (position, step size, RNG counter), on the oracle, so that a decision the two
+    take differently inside the margin below does not send the rest of the comparison down two
+    different chains.
 
-    The log accept ratio is a sum over 58368 rows at the end of a 1000-step trajectory; FP32 rounding
-    differences of the gradient (1e-7 relative) grow along it, the more the larger the energy error of
-    the trajectory is.  Over several builds of the kernel (each takes the burn-in a different way, so
-    each starts this leg from another state) the two implementations differed by up to 0.15 in it where
-    it is of order 1 and by up to 0.19 where it is of order 6, and never in a decision.  The tolerance
-    is TOL = 0.25 + 0.1 |log alpha|: the two values must agree to TOL, decisions must agree wherever the
-    uniform is further than TOL from the oracle's ratio, how many transitions fall inside that margin
-    is reported, and at most two of the 20 may disagree in all."""
+    The log accept ratio is a sum over 58368 rows at the end of a 1000-step trajectory, and a
+    trajectory of this posterior amplifies rounding: started one ulp away in every weight, the oracle
+    itself returns a log accept ratio that differs by about 0.1 (rms; measured 0.115), which is also
+    how far the GPU is from it (0.113), while a float64 trajectory lies between them (GPU 0.06 from
+    it, oracle 0.09).  So the bounds are stated against that sensitivity, measured in the test:
+      a. rms |GPU - oracle| over the 20 transitions <= 2 rms |oracle(+1 ulp) - oracle| + 0.02;
+      b. over the first 6 transitions, rms |GPU - float64| <= 2.5 rms |oracle - float64| + 0.03;
+      c. no transition differs by more than 1 + 0.2 |log alpha| (a missing term or row range);
+      d. decisions agree wherever the uniform is further from the oracle's ratio than the margin
+         0.3 + 0.1 |log alpha| + 2 |oracle(+1 ulp) - oracle|; at least 10 of the 20 are that clear,
+         and at most 3 decisions differ in all."""
     c = config0_chain
-    s, st = c["s"], c["state"]
-    assert st["transitions_done"] == 100
-    s.run(20)
-    tr = s.get_traces(0)
+    s = c["s"]
+    assert c["state"]["transitions_done"] == 100
+    eps_adapted = np.float32(c["state"]["eps"])
+    n_tr, n_f64 = 20, 6
+    la_gpu, la_ref, la_pert, la_f64 = np.zeros(n_tr), np.zeros(n_tr), np.zeros(n_tr), np.zeros(n_f64)
+    acc_gpu, acc_ref = np.zeros(n_tr, dtype=np.int64), np.zeros(n_tr, dtype=np.int64)
     t0 = time.time()
-    ref = orc.run_chain_from(c["om"], c["oh"], c["X"], c["y"], st["w"], st["eps"], 100, 20)
-    say("oracle: 20 full-length transitions in %.1f s" % (time.time() - t0))
-    lu = np.array([orc.log_uniform(0, 0, 100 + k) for k in range(20)])
-    la_gpu, la_ref = tr["log_acpt"][100:120], ref["log_acpt"]
-    acc_gpu, acc_ref = tr["accept"][100:120], ref["accept"]
-    tol = 0.25 + 0.1 * np.abs(la_ref)
-    clear = np.abs(lu - la_ref) > tol
-    say("adapted leg: %d of 20 transitions inside the margin; max |log alpha gpu - oracle| / tolerance = %.2f; "
-        "accepted gpu %d, oracle %d" % ((~clear).sum(), (np.abs(la_gpu - la_ref) / tol).max(), acc_gpu.sum(),
-                                         acc_ref.sum()))
-    for k in range(20):
-        say("  t=%d log u %.4f  log alpha gpu %.4f oracle %.4f  accept %d %d" % (
-            100 + k, lu[k], la_gpu[k], la_ref[k], acc_gpu[k], acc_ref[k]))
+    for k in range(n_tr):
+        st = s.get_chain_state(0)
+        assert st["transitions_done"] == 100 + k and np.float32(st["eps"]) == eps_adapted
+        s.run(1)
+        tr = s.get_traces(0)
+        w = np.asarray(st["w"], dtype=np.float32)
+        ref = orc.run_chain_from(c["om"], c["oh"], c["X"], c["y"], w, st["eps"], 100 + k, 1)
+        w_up = np.nextafter(w, np.float32(np.inf)).astype(np.float32)
+        pert = orc.run_chain_from(c["om"], c["oh"], c["X"], c["y"], w_up, st["eps"], 100 + k, 1)
+        la_gpu[k], acc_gpu[k] = tr["log_acpt"][100 + k], tr["accept"][100 + k]
+        la_ref[k], acc_ref[k] = ref["log_acpt"][0], ref["accept"][0]
+        la_pert[k] = pert["log_acpt"][0]
+        if k < n_f64:
+            la_f64[k] = _log_alpha_f64(orc, c["X"], c["y"], w, st["eps"], 100 + k)
+            say("  t=%d float64 trajectory done (%.0f s so far)" % (100 + k, time.time() - t0))
+    say("20 transitions: GPU, oracle twice, float64 for the first %d, in %.0f s" % (n_f64, time.time() - t0))
+    lu = np.array([orc.log_uniform(0, 0, 100 + k) for k in range(n_tr)])
+    margin = 0.3 + 0.1 * np.abs(la_ref) + 2.0 * np.abs(la_pert - la_ref)
+    clear = np.abs(lu - la_ref) > margin
+    for k in range(n_tr):
+        say("  t=%d log u %.4f  log alpha gpu %.4f oracle %.4f oracle(+1ulp) %.4f%s  accept %d %d" % (
+            100 + k, lu[k], la_gpu[k], la_ref[k], la_pert[k],
+            "  float64 %.4f" % la_f64[k] if k < n_f64 else "", acc_gpu[k], acc_ref[k]))
+    rms_gpu, rms_pert = _rms(la_gpu - la_ref), _rms(la_pert - la_ref)
+    rms_gpu64, rms_ref64 = _rms(la_gpu[:n_f64] - la_f64), _rms(la_ref[:n_f64] - la_f64)
+    say("adapted leg: rms |gpu - oracle| %.4f, |oracle(+1ulp) - oracle| %.4f; against float64: gpu %.4f, oracle %.4f; "
+        "%d of 20 inside the margin; accepted gpu %d, oracle %d" % (
+            rms_gpu, rms_pert, rms_gpu64, rms_ref64, (~clear).sum(), acc_gpu.sum(), acc_ref.sum()))
     assert np.all(np.isfinite(la_gpu)) and np.all(np.isfinite(la_ref))
-    assert np.array_equal(acc_gpu[clear], acc_ref[clear])
-    assert clear.sum() >= 12, "too few transitions outside the margin to say anything"
-    assert (acc_gpu != acc_ref).sum() <= 2
-    assert np.all(np.abs(la_gpu - la_ref) < tol)
-    assert acc_ref.sum() >= 3                                 # an adapted chain does accept
+    assert rms_gpu <= 2.0 * rms_pert + 0.02                                   # a
+    assert rms_gpu64 <= 2.5 * rms_ref64 + 0.03                                # b
+    assert bool(np.all(np.abs(la_gpu - la_ref) <= 1.0 + 0.2 * np.abs(la_ref)))  # c
+    assert np.array_equal(acc_gpu[clear], acc_ref[clear])                     # d
+    assert clear.sum() >= 10, "too few transitions outside the margin to say anything"
+    assert (acc_gpu != acc_ref).sum() <= 3
+    assert acc_gpu.sum() >= 3                                 # an adapted chain does accept
     # the step size no longer changes after the burn-in
-    assert np.all(tr["eps"][100:120] == np.float32(st["eps"]))
+    assert np.all(s.get_traces(0)["eps"][100:120] == eps_adapted)
 
 
 # ------------------------------------------------------------------------------------------------
