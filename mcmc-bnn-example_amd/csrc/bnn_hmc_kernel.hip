@@ -256,7 +256,11 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   cx.x_vec_ok = a.x_vec_ok != 0;
   cx.y_vec_ok = a.y_vec_ok != 0;
   {
-    const int gw = rank * W + wave, GW = a.G * W;
+    // The rows go to the waves in equal contiguous runs of tiles, the remainder spread evenly along
+    // the run order.  Waves w and w + W / 2 share a SIMD: they take neighbouring runs, so that when the
+    // tile count does not divide no SIMD gets two of the longer runs while another gets two short ones.
+    const int pos = W == 8 ? ((wave & 3) * 2 + (wave >> 2)) : wave;
+    const int gw = rank * W + pos, GW = a.G * W;
     cx.tile_begin = (int)((long)a.n_tiles * gw / GW);
     cx.tile_end = (int)((long)a.n_tiles * (gw + 1) / GW);
   }
