@@ -43,9 +43,9 @@ def main(out):
     if kt:
         durs = [(int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e6
                 for r in csv.DictReader(open(kt)) if "hmc_kernel" in r["Kernel_Name"]]
-        # launches of transitions take tens of milliseconds and more; the bootstrap and state
-        # evaluations that precede them well under one
-        trans = [d for d in durs if d > 5.0]
+        # launches of transitions take a hundred milliseconds and more (the tail batch of a 200-window
+        # run a sixth of a full batch); the bootstrap and state evaluations that precede them a few at most
+        trans = [d for d in durs if d > 0.05 * max(durs)]
         lines.append("hmc_kernel dispatches: %d evaluation launches (%.3f ms in all), %d launches of "
                      "transitions: %s ms" % (len(durs) - len(trans), sum(durs) - sum(trans), len(trans),
                                              ", ".join("%.1f" % d for d in trans)))
