@@ -239,8 +239,14 @@ int make_plan(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& 
 
 // Exchange scratch: partial records for `wgs` co-resident workgroups (double-buffered), one totals
 // record and one barrier line per chain group (at most `groups`), status words.
-size_t workspace_bytes_for(int P, int wgs, int groups) {
-  const size_t slot = (size_t)partial_slot_floats(P);
+// Floats per partial record.  The 64 -> 128 -> 1 kernel exchanges plain floats behind a barrier; the
+// 22 -> 40 -> 1 kernel exchanges flagged 8-byte packets (value, step number) that are polled directly.
+size_t exchange_slot_floats(int P, bool wide) {
+  return (size_t)partial_slot_floats(P) * (wide ? 1 : 2);
+}
+
+size_t workspace_bytes_for(int P, int wgs, int groups, bool wide) {
+  const size_t slot = exchange_slot_floats(P, wide);
   size_t bytes = STATUS_WORDS * sizeof(unsigned);
   bytes += (size_t)(wgs + 31) / 32 * 32 * sizeof(unsigned long long);
   bytes += (size_t)wgs * 2 * slot * sizeof(float);
@@ -257,11 +263,13 @@ struct Workspace {
   float* partials;
   float* totals;
   unsigned* barrier;
+  size_t slot_floats;
 };
-Workspace carve_workspace(void* base, int P, int wgs, int groups) {
+Workspace carve_workspace(void* base, int P, int wgs, int groups, bool wide) {
   Workspace w;
   char* b = (char*)base;
-  const size_t slot = (size_t)partial_slot_floats(P);
+  const size_t slot = exchange_slot_floats(P, wide);
+  w.slot_floats = slot;
   w.status = (unsigned*)b;
   b += STATUS_WORDS * sizeof(unsigned);
   w.rank_hash = (unsigned long long*)b;
@@ -272,6 +280,17 @@ Workspace carve_workspace(void* base, int P, int wgs, int groups) {
   b += (size_t)groups * slot * sizeof(float);
   w.barrier = (unsigned*)b;
   return w;
+}
+
+// What a launch of `groups` chain groups of G workgroups needs cleared beforehand: the barrier counters
+// (64 -> 128 -> 1) or the flags of the packets it will poll (22 -> 40 -> 1: step numbers restart at 1
+// with every launch, so no packet of an earlier launch may survive).
+hipError_t clear_exchange(const Workspace& w, const KArgs& a, int groups, bool wide, hipStream_t st) {
+  if (wide) return launch_fill_u32(w.barrier, (size_t)groups * BARRIER_STRIDE_WORDS, 0u, st);
+  hipError_t rc = launch_fill_u32((unsigned*)w.partials, (size_t)groups * 2 * a.G * w.slot_floats, 0u, st);
+  if (rc == hipSuccess && a.two_phase)
+    rc = launch_fill_u32((unsigned*)w.totals, (size_t)groups * w.slot_floats, 0u, st);
+  return rc;
 }
 
 // Synchronises `stream` and reads the status words the launches on it have left since the words
@@ -514,7 +533,7 @@ KArgs base_args(const bnnhmc_sampler* s) {
   a.debug_drop_rank = debug_drop_rank();
   a.debug_perturb_hash_rank = debug_perturb_hash_rank();
   a.balance = env_balance();
-  Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups);
+  Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups, s->plan.wide);
   a.partials = w.partials;
   a.totals = w.totals;
   a.barrier = w.barrier;
@@ -528,7 +547,8 @@ int launch_and_count(bnnhmc_sampler* s, KArgs& a, int groups) {
   int wgs = 0;
   set_grid(a, groups, s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs, 256) : s->plan.G,
            &wgs);
-  HIP_TRY(launch_fill_u32(a.barrier, (size_t)groups * BARRIER_STRIDE_WORDS, 0u, s->stream));
+  HIP_TRY(clear_exchange(carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups, s->plan.wide),
+                         a, groups, s->plan.wide, s->stream));
   HIP_TRY(launch_hmc_kernel(s->plan.kernel, a, wgs, s->plan.threads, s->plan.dyn_lds, s->stream));
   HIP_TRY(launch_compare_hashes(a.rank_hash, wgs, a.G, a.status, s->stream));
   s->last_workgroups = wgs;
@@ -702,7 +722,7 @@ size_t bnnhmc_step_workspace_bytes(const bnnhmc_model* model, const bnnhmc_launc
   if (!model) return 0;
   // sized for the default group (256) when none is configured, whatever device is present
   const int G = launch && launch->cus_per_chain > 0 ? launch->cus_per_chain : 256;
-  return workspace_bytes_for(make_layout(model->d0, model->d1).P, G, 1);
+  return workspace_bytes_for(make_layout(model->d0, model->d1).P, G, 1, model->d0 == 64 && model->d1 == 128);
 }
 
 // The step operator on a given exchange scratch; allocates nothing (device and plan queries happen on
@@ -731,9 +751,9 @@ static int mcmc_step_on(const bnnhmc_model* model, const bnnhmc_launch* launch, 
   if (G > plan.resident_wgs)
     return fail(BNNHMC_ERR_RESIDENCY, "%d workgroups per chain requested but only %d can be resident", G,
                 plan.resident_wgs);
-  if (workspace_bytes < workspace_bytes_for(L.P, G, 1))
+  if (workspace_bytes < workspace_bytes_for(L.P, G, 1, plan.wide))
     return fail(BNNHMC_ERR_INVALID, "workspace too small: %zu < %zu bytes", workspace_bytes,
-                workspace_bytes_for(L.P, G, 1));
+                workspace_bytes_for(L.P, G, 1, plan.wide));
   hipStream_t st = (hipStream_t)stream;
   KArgs a;
   memset(&a, 0, sizeof(a));
@@ -763,7 +783,7 @@ static int mcmc_step_on(const bnnhmc_model* model, const bnnhmc_launch* launch, 
   a.debug_drop_rank = debug_drop_rank();
   a.debug_perturb_hash_rank = debug_perturb_hash_rank();
   a.balance = env_balance();
-  Workspace w = carve_workspace(workspace, L.P, G, 1);
+  Workspace w = carve_workspace(workspace, L.P, G, 1, plan.wide);
   a.partials = w.partials;
   a.totals = w.totals;
   a.barrier = w.barrier;
@@ -771,9 +791,9 @@ static int mcmc_step_on(const bnnhmc_model* model, const bnnhmc_launch* launch, 
   a.rank_hash = w.rank_hash;
   int wgs = 0;
   set_grid(a, 1, G, &wgs);
-  // status and barrier words start from zero on every call
+  // status words and the exchange area start from zero on every call
   HIP_TRY(launch_fill_u32(w.status, STATUS_WORDS, 0u, st));
-  HIP_TRY(launch_fill_u32(w.barrier, BARRIER_STRIDE_WORDS, 0u, st));
+  HIP_TRY(clear_exchange(w, a, 1, plan.wide, st));
   HIP_TRY(launch_hmc_kernel(plan.kernel, a, wgs, plan.threads, plan.dyn_lds, st));
   HIP_TRY(launch_compare_hashes(a.rank_hash, wgs, G, a.status, st));
   return BNNHMC_OK;
@@ -914,7 +934,7 @@ int bnnhmc_create(const bnnhmc_model* model, const bnnhmc_hmc* hmc, const bnnhmc
   }
   const size_t C = s->n_chains;
   const int eval_groups_max = s->plan.max_groups;
-  s->workspace_bytes = workspace_bytes_for(s->L.P, s->plan.resident_wgs, s->plan.max_groups);
+  s->workspace_bytes = workspace_bytes_for(s->L.P, s->plan.resident_wgs, s->plan.max_groups, s->plan.wide);
   char* ws = nullptr;
   if ((rc = s->alloc(&s->X, (size_t)n_windows * model->n * model->d0)) ||
       (rc = s->alloc(&s->y, (size_t)n_windows * s->n_pad)) ||

@@ -230,7 +230,12 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   // start momentum of the running transition, and the thread's state hash
   __shared__ float s_wc[PPT * T], s_gc[PPT * T], s_m0[PPT * T];
   __shared__ unsigned long long s_hacc[T];
-  __shared__ int s_flag;
+  __shared__ int s_flag[2];  // by step parity: cleared by a thread that abandoned a wait
+  // stage 2: the sums over the records (own array: the waves' slots may still be being read by stage 1
+  // of a slower wave), the reducers' per-wave slice sums, the log-likelihood difference
+  __shared__ float s_sum[P_AL];
+  __shared__ float s_red2[W][32];
+  __shared__ double s_dl;
 
   // ---- which chain group, which rank inside it ----
   int lin = blockIdx.x;
@@ -272,8 +277,8 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   cx.partner = wave ^ (W / 2);
 
   const ModelConsts mc = a.mc;
-  float* part_base = a.partials + (size_t)group * 2 * a.G * SLOT;
-  unsigned* counter = a.barrier + (size_t)group * BARRIER_STRIDE_WORDS;
+  // records of flagged packets (8 bytes per parameter), two per workgroup (by step parity)
+  unsigned long long* part_base = reinterpret_cast<unsigned long long*>(a.partials) + (size_t)group * 2 * a.G * SLOT;
   unsigned bar_epoch = 0;
   int buf = 0;
 
@@ -368,6 +373,8 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         }
       }
       if ((tid & 63) == 0) s_progress[wave] = 0;
+      const unsigned epoch = bar_epoch + 1;  // the steps of this launch from 1
+      if (tid == 0) s_flag[epoch & 1] = 1;
       __syncthreads();
       BNN_PHASE(0)  // update + sync
       layer.template load_weights<LIK>(s_w, mc);
@@ -385,162 +392,165 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       layer.template write_partials<LIK>(s_slots[wave], s_w, last);
       __syncthreads();
       BNN_PHASE(3)  // wave partials -> LDS + sync
-      // ---- stage 1: fixed-order sum over this workgroup's waves -> global partial record ----
-      float* my_part = part_base + ((size_t)buf * a.G + rank) * SLOT;
-#pragma unroll
-      for (int i = 0; i < PPT; ++i) {
-        const int p = tid + i * T;
-        if (p < P) {
-          float v = s_slots[0][p];
-#pragma unroll
-          for (int wv = 1; wv < W; ++wv) v += s_slots[wv][p];
-          st_agent(my_part + p, v);
-        }
-      }
-      if (last && tid == 0) {
-        double d = 0.0;
-#pragma unroll
-        for (int wv = 0; wv < W; ++wv) {
-          const uint64_t bits = ((uint64_t)__builtin_bit_cast(uint32_t, s_slots[wv][P_AL + 1]) << 32) |
-                                __builtin_bit_cast(uint32_t, s_slots[wv][P_AL]);
-          d += bits_to_double(bits);
-        }
-        const uint64_t bits = double_to_bits(d);
-        st_agent(my_part + P_AL, __builtin_bit_cast(float, (uint32_t)bits));
-        st_agent(my_part + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)));
-      }
-      BNN_PHASE(4)  // stage 1 + global store
-      // two-phase reduction: only the workgroups that reduce a slice need the others' records now
-      constexpr int N_RED = (P + 31) / 32;
-      const bool reducer = rank < N_RED;
-      ok = group_barrier(counter, a.G, rank, ++bar_epoch, a.status, a.spin_limit, &s_flag,
-                         rank != a.debug_drop_rank, !a.two_phase || reducer);
-      if (!ok) break;
-      BNN_PHASE(5)  // group barrier
-      const float* grp_part = part_base + (size_t)buf * a.G * SLOT;
-      if (!a.two_phase) {
-        // ---- stage 2 (small groups): every workgroup adds the G records.  A thread takes one 16-byte
-        //      column of the records and every H-th record (H = T / 256 thread sets), eight loads in
-        //      flight, records in ascending order; the sets are then added in a fixed order through
-        //      LDS, seeded with the prior gradient as block 0 does in the reference
-        //      (mcmc_step_ffma.h:144) ----
-        constexpr int NCOL = P_AL / 4, CW = 256, H = T / CW;
-        static_assert(NCOL <= CW && T % CW == 0 && H <= W, "stage 2 thread sets");
-        {
-          const int col = tid & (CW - 1), part = tid / CW;  // part is uniform within a wave
-          if (col < NCOL) {
-            f4 v = {0.f, 0.f, 0.f, 0.f};
-            const float* src = grp_part + 4 * col;
-            for (int r0 = part; r0 < a.G; r0 += 8 * H) {
-              f4 t8[8];
-              const float* p8[8];
-#pragma unroll
-              for (int k = 0; k < 8; ++k) p8[k] = src + (size_t)min(r0 + H * k, a.G - 1) * SLOT;
-              ld_agent4x8(t8, p8);
-#pragma unroll
-              for (int k = 0; k < 8; ++k)
-                if (r0 + H * k < a.G) v += t8[k];  // wave-uniform condition
-            }
-            // rows 0 .. H-1 of s_slots are free: stage 1 read them before the barrier
-            *reinterpret_cast<f4*>(&s_slots[part][4 * col]) = v;
-          }
-          __syncthreads();
-#pragma unroll
-          for (int i = 0; i < PPT; ++i) {
-            const int p = tid + i * T;
-            if (p < P) {
-              float v = prior_grad(mc, w[i]);
-#pragma unroll
-              for (int h = 0; h < H; ++h) v += s_slots[h][p];
-              g[i] = v;
-            }
-          }
-        }
-        if (last) {
-          double d = 0.0;
-          for (int r = 0; r < a.G; ++r) {
-            const float lo = ld_agent(grp_part + (size_t)r * SLOT + P_AL);
-            const float hi = ld_agent(grp_part + (size_t)r * SLOT + P_AL + 1);
-            d += bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
-                                __builtin_bit_cast(uint32_t, lo));
-          }
-          dl_total = d;
-        }
-      } else {
-        // ---- stage 2 (large groups), in two phases.  Phase 1: workgroup `rank` < ceil(P / 32)
-        //      reduces the 32-parameter slice [32 rank, 32 rank + 32) -- one 128-byte line of every
-        //      record, so that no fetched line is mostly unused -- over all G records: thread
-        //      (record lane rl = tid / 8, 16-byte column c = tid % 8) adds records rl, rl + T/8, ...
-        //      in order, the record lanes of a wave are added by a fixed xor tree and the waves in
-        //      order through LDS.  Phase 2 (once all reducing workgroups have stored their slices):
-        //      everyone reads the totals.  Workgroups that reduce nothing do not wait for the first
-        //      barrier at all. ----
-        float* tot = a.totals + (size_t)group * SLOT;
-        constexpr int RL = T / 8;  // record lanes of a workgroup
-        if (reducer) {
-          const int c = tid & 7, rl = tid >> 3;
-          const float* src = grp_part + 32 * rank + 4 * c;
-          f4 v = {0.f, 0.f, 0.f, 0.f};
-          for (int r0 = rl; r0 < a.G; r0 += 8 * RL) {
-            f4 t8[8];
-            const float* p8[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) p8[k] = src + (size_t)min(r0 + RL * k, a.G - 1) * SLOT;
-            ld_agent4x8(t8, p8);
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-              if (r0 + RL * k < a.G) v += t8[k];
-          }
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float x = v[e];
-            x += __shfl_xor(x, 8);
-            x += __shfl_xor(x, 16);
-            x += __shfl_xor(x, 32);
-            v[e] = x;
-          }
-          // rows of s_slots are free: stage 1 read them before the barrier
-          if ((tid & 63) < 8) *reinterpret_cast<f4*>(&s_slots[wave][4 * c]) = v;
-        }
-        __syncthreads();
-        if (reducer && tid < 32 && 32 * rank + tid < P) {
-          float x = s_slots[0][tid];
-#pragma unroll
-          for (int wv = 1; wv < W; ++wv) x += s_slots[wv][tid];
-          st_agent(tot + 32 * rank + tid, x);
-        }
-        if (last && rank == N_RED - 1 && wave == W - 1) {
-          const int lane = tid & 63;
-          double d = 0.0;
-          for (int r = lane; r < a.G; r += 64) {
-            const float lo = ld_agent(grp_part + (size_t)r * SLOT + P_AL);
-            const float hi = ld_agent(grp_part + (size_t)r * SLOT + P_AL + 1);
-            d += bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
-                                __builtin_bit_cast(uint32_t, lo));
-          }
-#pragma unroll
-          for (int msk = 1; msk < 64; msk <<= 1) d += shfl_xor_d(d, msk);
-          if (lane == 0) {
-            const uint64_t bits = double_to_bits(d);
-            st_agent(tot + P_AL, __builtin_bit_cast(float, (uint32_t)bits));
-            st_agent(tot + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)));
-          }
-        }
-        ok = reducer_barrier(counter, N_RED, reducer, rank, bar_epoch, a.status, a.spin_limit, &s_flag,
-                             rank != a.debug_drop_rank);
-        if (!ok) break;
+      // ---- stage 1: fixed-order sum over this workgroup's waves -> the workgroup's record of flagged
+      //      packets (see st_packet); the padding up to P_AL is written too, so that every 16-byte column
+      //      a reader polls is complete ----
+      ++bar_epoch;
+      unsigned long long* my_part = part_base + ((size_t)buf * a.G + rank) * SLOT;
+      if (rank != a.debug_drop_rank) {
 #pragma unroll
         for (int i = 0; i < PPT; ++i) {
           const int p = tid + i * T;
-          if (p < P) g[i] = prior_grad(mc, w[i]) + ld_agent(tot + p);
+          if (p < P_AL) {
+            float v = 0.0f;
+            if (p < P) {
+              v = s_slots[0][p];
+#pragma unroll
+              for (int wv = 1; wv < W; ++wv) v += s_slots[wv][p];
+            }
+            st_packet(my_part + p, v, epoch);
+          }
         }
-        if (last) {
-          const float lo = ld_agent(tot + P_AL);
-          const float hi = ld_agent(tot + P_AL + 1);
-          dl_total = bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
-                                    __builtin_bit_cast(uint32_t, lo));
+        if (last && tid == 0) {
+          double d = 0.0;
+#pragma unroll
+          for (int wv = 0; wv < W; ++wv) {
+            const uint64_t bits = ((uint64_t)__builtin_bit_cast(uint32_t, s_slots[wv][P_AL + 1]) << 32) |
+                                  __builtin_bit_cast(uint32_t, s_slots[wv][P_AL]);
+            d += bits_to_double(bits);
+          }
+          const uint64_t bits = double_to_bits(d);
+          st_packet(my_part + P_AL, __builtin_bit_cast(float, (uint32_t)bits), epoch);
+          st_packet(my_part + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)), epoch);
         }
       }
+      BNN_PHASE(4)  // stage 1 + global store
+      BNN_PHASE(5)  // (no barrier: the records are polled)
+      const unsigned long long* grp_part = part_base + (size_t)buf * a.G * SLOT;
+      bool fine = true;  // cleared by a thread whose wait was abandoned
+      // the log-likelihood difference of the records, in record order per lane and a fixed tree over
+      // the lanes (last step only; one wave)
+      auto sum_dl = [&]() {
+        const int lane = tid & 63;
+        double d = 0.0;
+        for (int r = lane; r < a.G; r += 64) {
+          const float lo = wait_packet(grp_part + (size_t)r * SLOT + P_AL, epoch, a.status, a.spin_limit, fine);
+          const float hi = wait_packet(grp_part + (size_t)r * SLOT + P_AL + 1, epoch, a.status, a.spin_limit, fine);
+          d += bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
+                              __builtin_bit_cast(uint32_t, lo));
+        }
+#pragma unroll
+        for (int msk = 1; msk < 64; msk <<= 1) d += shfl_xor_d(d, msk);
+        return d;
+      };
+      constexpr int N_RED = (P_AL + 31) / 32;
+      if (!a.two_phase) {
+        // ---- stage 2 (small groups): every workgroup adds the G records.  A thread takes 16-byte
+        //      columns (two parameters) of the records, eight loads in flight, records in ascending
+        //      order, polling until all of them are this step's; the prior gradient is added as block 0
+        //      does in the reference (mcmc_step_ffma.h:144) ----
+        constexpr int NCOL = P_AL / 2;
+        for (int col = tid; col < NCOL; col += T) {
+          float v0 = 0.0f, v1 = 0.0f;
+          const unsigned long long* src = grp_part + 2 * col;
+          for (int r0 = 0; r0 < a.G; r0 += 8) {
+            f4 t8[8];
+            const unsigned long long* p8[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) p8[k] = src + (size_t)min(r0 + k, a.G - 1) * SLOT;
+            wait_packets4x8(t8, p8, a.G - r0, epoch, a.status, a.spin_limit, fine);
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+              if (r0 + k < a.G) {  // wave-uniform condition
+                v0 += t8[k][0];
+                v1 += t8[k][2];
+              }
+          }
+          s_sum[2 * col] = v0;
+          s_sum[2 * col + 1] = v1;
+        }
+        if (last && wave == W - 1) {
+          const double d = sum_dl();
+          if ((tid & 63) == 0) s_dl = d;
+        }
+      } else {
+        // ---- stage 2 (large groups), in two phases.  Phase 1: workgroup `rank` < ceil(P / 32) reduces
+        //      the 32-parameter slice [32 rank, 32 rank + 32) -- 256 bytes of every record -- over all
+        //      G records: thread (record lane rl = tid / 16, 16-byte column c = tid % 16) adds records
+        //      rl, rl + T/16, ... in order, the record lanes of a wave are added by a fixed xor tree and
+        //      the waves in order through LDS; the totals go out as flagged packets.  Phase 2: everyone
+        //      polls the totals. ----
+        unsigned long long* tot = reinterpret_cast<unsigned long long*>(a.totals) + (size_t)group * SLOT;
+        constexpr int RL = T / 16;  // record lanes of a workgroup
+        const bool reducer = rank < N_RED;
+        if (reducer) {
+          const int c = tid & 15, rl = tid >> 4;
+          const bool col_ok = 32 * rank + 2 * c < P_AL;  // P_AL is even: a column is whole or absent
+          const unsigned long long* src = grp_part + 32 * rank + 2 * c;
+          float v0 = 0.0f, v1 = 0.0f;
+          for (int r0 = rl; r0 < a.G; r0 += 8 * RL) {
+            f4 t8[8];
+            const unsigned long long* p8[8];
+            int valid = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+              p8[k] = src + (size_t)min(r0 + RL * k, a.G - 1) * SLOT;
+              if (r0 + RL * k < a.G) valid = k + 1;
+            }
+            wait_packets4x8(t8, p8, col_ok ? valid : 0, epoch, a.status, a.spin_limit, fine);
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+              if (k < valid) {
+                v0 += t8[k][0];
+                v1 += t8[k][2];
+              }
+          }
+          v0 += __shfl_xor(v0, 16);
+          v0 += __shfl_xor(v0, 32);
+          v1 += __shfl_xor(v1, 16);
+          v1 += __shfl_xor(v1, 32);
+          if ((tid & 63) < 16) {
+            s_red2[wave][2 * c] = v0;
+            s_red2[wave][2 * c + 1] = v1;
+          }
+        }
+        __syncthreads();
+        if (reducer && tid < 32 && 32 * rank + tid < P_AL && rank != a.debug_drop_rank) {
+          float x = s_red2[0][tid];
+#pragma unroll
+          for (int wv = 1; wv < W; ++wv) x += s_red2[wv][tid];
+          st_packet(tot + 32 * rank + tid, x, epoch);
+        }
+        if (last && rank == N_RED - 1 && wave == W - 1) {
+          const double d = sum_dl();
+          if ((tid & 63) == 0) {
+            const uint64_t bits = double_to_bits(d);
+            st_packet(tot + P_AL, __builtin_bit_cast(float, (uint32_t)bits), epoch);
+            st_packet(tot + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)), epoch);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < PPT; ++i) {
+          const int p = tid + i * T;
+          if (p < P) s_sum[p] = wait_packet(tot + p, epoch, a.status, a.spin_limit, fine);
+        }
+        if (last && tid == 0) {
+          const float lo = wait_packet(tot + P_AL, epoch, a.status, a.spin_limit, fine);
+          const float hi = wait_packet(tot + P_AL + 1, epoch, a.status, a.spin_limit, fine);
+          s_dl = bits_to_double(((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32) |
+                                __builtin_bit_cast(uint32_t, lo));
+        }
+      }
+      if (!fine) s_flag[epoch & 1] = 0;
+      __syncthreads();
+      ok = s_flag[epoch & 1] != 0;
+      if (!ok) break;
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        const int p = tid + i * T;
+        if (p < P) g[i] = prior_grad(mc, w[i]) + s_sum[p];
+      }
+      if (last) dl_total = s_dl;
       buf ^= 1;
       BNN_PHASE(6)  // stage 2
     }

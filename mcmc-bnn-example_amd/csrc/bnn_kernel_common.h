@@ -230,6 +230,74 @@ __device__ __forceinline__ int poll_counter(unsigned* line, unsigned target, uns
   return 1;
 }
 
+// ------------------------------------------------------------------------------------------------
+// Flagged packets: the exchange of the 22 -> 40 -> 1 kernel needs no barrier.  A value travels as
+// 8 bytes {value, flag}, written by one 8-byte store, so it arrives whole; the flag is the number of the
+// leapfrog step within the launch (from 1; the host zeroes the exchange area before every launch), and
+// a reader polls the packet itself until the flag says it is this step's.  One memory round trip per
+// hand-off instead of three (store, counter, load).  Bounded like the barrier: after spin_limit polls,
+// or when another workgroup has given up, the reader gives up (status[0] set) and the launch is abandoned.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void st_packet(unsigned long long* p, float v, unsigned flag) {
+  __hip_atomic_store(p, ((unsigned long long)flag << 32) | (unsigned long long)__builtin_bit_cast(unsigned, v),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long ld_packet(const unsigned long long* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// bookkeeping of one more poll; false when the launch is being abandoned
+__device__ __forceinline__ bool poll_again(unsigned& polls, unsigned* status, unsigned spin_limit) {
+  __builtin_amdgcn_s_sleep(1);
+  if ((++polls & 63u) == 0u) {
+    if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return false;
+    if (polls >= spin_limit) {
+      __hip_atomic_store(status + 1, (unsigned)blockIdx.x + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return false;
+    }
+  }
+  return true;
+}
+// the value of one packet once its flag is `flag`; `fine` is cleared when the wait is abandoned
+__device__ __forceinline__ float wait_packet(const unsigned long long* p, unsigned flag, unsigned* status,
+                                             unsigned spin_limit, bool& fine) {
+  unsigned polls = 0;
+  unsigned long long v = ld_packet(p);
+  while ((unsigned)(v >> 32) != flag) {
+    if (!poll_again(polls, status, spin_limit)) {
+      fine = false;
+      break;
+    }
+    v = ld_packet(p);
+  }
+  return __builtin_bit_cast(float, (unsigned)v);
+}
+// (taken by value: applied straight to an element of a vector, __builtin_bit_cast reads element 0)
+__device__ __forceinline__ unsigned float_bits(float f) { return __builtin_bit_cast(unsigned, f); }
+// Eight 16-byte columns (two packets each) of up to eight records, polled until every packet of the
+// first `valid` records carries `flag`.
+__device__ __forceinline__ void wait_packets4x8(f4 (&t)[8], const unsigned long long* const (&p)[8], int valid,
+                                                unsigned flag, unsigned* status, unsigned spin_limit,
+                                                bool& fine) {
+  const float* q[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) q[k] = reinterpret_cast<const float*>(p[k]);
+  unsigned polls = 0;
+  for (;;) {
+    ld_agent4x8(t, q);
+    bool ok = true;
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (k < valid)
+        ok = ok && float_bits(t[k][1]) == flag && float_bits(t[k][3]) == flag;
+    if (ok) break;
+    if (!poll_again(polls, status, spin_limit)) {
+      fine = false;
+      break;
+    }
+  }
+}
+
 // `epoch` counts the barriers of this launch from 1.  Up to 64 workgroups add to the group's counter
 // directly.  Larger groups arrive in blocks of 32 ranks at a block counter and the last arriver of a
 // block adds to the group's counter: 256 same-address atomics cost 3.8 us, 32 + 8 cost 2.3 us.
