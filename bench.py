@@ -6,8 +6,8 @@ of the 22->40->1 Bayesian MLP, full batch of 58368 rows each (features ~ N(0,1),
 N(0, 0.01^2) noise, Gaussian likelihood, Gaussian weight prior), one chain per window, HMC with 1000
 leapfrog steps per transition, all 200 windows resident in HBM (1.07 GB).  A "step" is one HMC transition
 (momentum resampling, 1000 fused leapfrog gradient evaluations, log accept ratio, Metropolis decision,
-sample store) of every one of the 200 windows: the library runs them as three batches of 64 chains at 4
-workgroups per chain and a last batch of 8 chains at 32 workgroups per chain.  The warm-up transitions
+sample store) of every one of the 200 windows: the library runs them as batches of 128 chains at 2
+workgroups per chain, 64 chains at 4 and 8 chains at 32, each over all 256 compute units.  The warm-up transitions
 are the burn-in (nothing stored), the timed ones store their samples.  The metric is leapfrog gradient
 evaluations per second; the minutes for 200 windows x (100 burn-in + 800 samples) are 900 steps plus the
 bootstrap evaluation, and --full runs that whole job.
@@ -42,6 +42,31 @@ def measured_traffic(kernel_key):
             return float(json.load(f)[kernel_key]["bytes_per_grad_eval"])
     except (OSError, KeyError, ValueError, TypeError):
         return None
+
+
+def batch_plan(n_chains, resident_wgs, cus_per_chain, wide):
+    """[(chains, workgroups per chain)] of the launches that cover n_chains, as the library lays them out:
+    a fixed group size when one is configured (the 64->128->1 default is 4), otherwise the largest
+    power-of-two number of chains that is left and fits, spread over the whole device; a batch that
+    leaves compute units idle gets its groups doubled while they still fit."""
+    def widen(g, b):
+        while g * 2 * b <= resident_wgs and g * 2 <= 256:
+            g *= 2
+        return g
+    fixed = cus_per_chain or (4 if wide else 0)
+    out, left = [], n_chains
+    while left > 0:
+        if fixed:
+            b = min(left, max(1, resident_wgs // fixed))
+            g = fixed if cus_per_chain else widen(fixed, b)
+        else:
+            b = 1
+            while b * 2 <= min(left, resident_wgs):
+                b *= 2
+            g = widen(1, b)
+        out.append((b, g))
+        left -= b
+    return out
 
 
 def cpu_baseline(seconds, n_rows=N_ROWS, d0=D0, d1=D1):
@@ -118,10 +143,11 @@ def main():
     n_rows, d0, d1, cpw = (WIDE_ROWS, WIDE_D0, WIDE_D1, WIDE_CHAINS) if wide else (N_ROWS, D0, D1, 1)
     flop_per_eval = 4 * n_rows * d1 * (d0 + 1)
     wgs_per_cu = 1 if wide or layer != pkg.LAYER_MFMA else launch.wgs_per_cu
-    group = launch.cus_per_chain or 4
-    resident = max(1, (cus * wgs_per_cu) // group)          # chains in flight
-    n_windows = args.windows or (max(1, resident // cpw) if wide else 200)
+    resident_wgs = cus * wgs_per_cu
+    n_windows = args.windows or (max(1, resident_wgs // 4 // cpw) if wide else 200)
     n_chains = n_windows * cpw
+    plan = batch_plan(n_chains, resident_wgs, launch.cus_per_chain, wide)
+    resident = plan[0][0]                                   # chains in flight in the first launches
 
     model = lib.default_model(d0=d0, d1=d1, n=n_rows, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01,
                               prior_scale=0.1)
@@ -206,7 +232,8 @@ def main():
                         "= one transition of every window, samples stored in the timed region" % (
                             4 if wide else 2, n_windows, cpw, min(n_chains, resident), d0, d1, n_rows, d0,
                             args.leapfrog),
-            "layer": args.layer, "cus_per_chain": group, "wgs_per_cu": wgs_per_cu,
+            "layer": args.layer, "wgs_per_cu": wgs_per_cu,
+            "launches_chains_x_workgroups_per_chain": ", ".join("%d x %d" % bg for bg in plan),
             "workgroups_last_launch": tm1["workgroups"], "compute_units": cus,
             "transitions_per_launch": args.transitions_per_launch,
             "eps0": float(hmc.eps0), "adapt_steps": int(hmc.adapt_steps),

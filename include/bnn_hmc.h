@@ -71,9 +71,11 @@ typedef struct bnnhmc_hmc {
 /* How the work is laid over the GPU.  Zero in a field selects the default. */
 typedef struct bnnhmc_launch {
   int layer;          /* BNNHMC_LAYER_MFMA (v_mfma_f32_16x16x4_f32) or BNNHMC_LAYER_FFMA          */
-  int cus_per_chain;  /* workgroups that share one chain's rows; 0 = default: 4 for a sampler (64   */
-                      /* chains in flight on 256 CUs; a smaller last batch is widened to fill the   */
-                      /* device, up to 256 per chain), 256 for the step operator                    */
+  int cus_per_chain;  /* workgroups that share one chain's rows; 0 = automatic.  Sampler,         */
+                      /* 22 -> 40 -> 1: batches of the largest power-of-two number of chains that  */
+                      /* is left and fits, each over the whole device (200 chains on 256 CUs: 128   */
+                      /* chains x 2 workgroups, 64 x 4, 8 x 32; one chain: 256); 64 -> 128 -> 1: 4, */
+                      /* a smaller last batch widened.  Step operator: 256                          */
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */
   int threads;        /* threads per workgroup; default 512 for MFMA (every tile loop), 256 for  */
                       /* FFMA and with wgs_per_cu = 2.  The plain MFMA loop is also built for    */

@@ -186,8 +186,12 @@ int make_plan_uncached(const bnnhmc_model& m, const bnnhmc_launch* lp, const Dev
   p.wgs_per_cu = std::min(per_cu, l.wgs_per_cu);
   const int resident = p.wgs_per_cu * di.cus;
   p.resident_wgs = resident;
-  // 0 = default: 4 workgroups per chain (64 chains in flight on 256 CUs)
-  p.G = l.cus_per_chain > 0 ? l.cus_per_chain : std::min(4, resident);
+  // 0 = automatic.  22 -> 40 -> 1: a batch is the largest power-of-two number of chains that is left
+  // and fits (one workgroup per chain at least), each chain on resident / batch workgroups -- 200
+  // chains on 256 CUs run as 128 x 2, 64 x 4, 8 x 32 (measured, evaluations/s with every CU busy:
+  // 2 workgroups per chain 386 k, 4: 379 k, 8: 368 k, 16: 341 k, 32: 289 k).  64 -> 128 -> 1: 4
+  // workgroups per chain, a last smaller batch widened.
+  p.G = l.cus_per_chain > 0 ? l.cus_per_chain : (p.wide ? std::min(4, resident) : 1);
   p.widen = l.cus_per_chain <= 0;
   if (p.G > resident)
     return fail(BNNHMC_ERR_RESIDENCY,
@@ -314,6 +318,19 @@ int read_status(void* workspace, hipStream_t stream) {
   return BNNHMC_OK;
 }
 
+// Chains of the next batch when `left` are still to run: as many as fit; with the automatic group size
+// of the 22 -> 40 -> 1 kernel the largest power of two of them, so that the batch fills the device with
+// equal groups (see make_plan_uncached).
+int batch_size(const Plan& p, int left) {
+  int groups = std::min(p.max_groups, left);
+  if (p.widen && !p.wide) {
+    int b = 1;
+    while (b * 2 <= groups) b *= 2;
+    groups = b;
+  }
+  return groups;
+}
+
 // Workgroups per chain for a batch of `groups` chains: the configured count, widened by powers of
 // two while the whole batch still fits the device (a last, smaller batch then uses every CU).
 int widen_group(int G, int groups, int resident_wgs, int cap) {
@@ -321,12 +338,15 @@ int widen_group(int G, int groups, int resident_wgs, int cap) {
   return G;
 }
 
-void set_grid(KArgs& a, int groups, int G, int* workgroups) {
+void set_grid(KArgs& a, int groups, int G, bool wide, int* workgroups) {
   const int wgs = groups * G;
   a.G = G;
-  // measured on MI355X: up to 64 workgroups per chain the single-barrier all-read reduction is
-  // faster than two barriers with small reads (a barrier that spans XCDs costs about 10 us)
-  a.two_phase = G > 64 ? 1 : 0;
+  // From 32 workgroups per chain on, each of the first 31 workgroups reduces one 32-parameter slice of
+  // the records and everyone reads the totals, instead of everyone reading every record.  Measured on
+  // MI355X with the 22 -> 40 -> 1 kernel (evaluations/s, all-read vs slices): G = 32: 278 k vs 288 k,
+  // G = 64: 183 k vs 230 k.  The 64 -> 128 -> 1 kernel, whose hand-offs go through barriers, switches
+  // above 64.
+  a.two_phase = G >= (wide ? 65 : 32) ? 1 : 0;
   a.n_groups = groups;
   a.xcd_map = (wgs % 8 == 0) && ((wgs / 8) % G == 0) ? 1 : 0;
   *workgroups = wgs;
@@ -546,7 +566,7 @@ KArgs base_args(const bnnhmc_sampler* s) {
 int launch_and_count(bnnhmc_sampler* s, KArgs& a, int groups) {
   int wgs = 0;
   set_grid(a, groups, s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs, 256) : s->plan.G,
-           &wgs);
+           s->plan.wide, &wgs);
   HIP_TRY(clear_exchange(carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups, s->plan.wide),
                          a, groups, s->plan.wide, s->stream));
   HIP_TRY(launch_hmc_kernel(s->plan.kernel, a, wgs, s->plan.threads, s->plan.dyn_lds, s->stream));
@@ -790,7 +810,7 @@ static int mcmc_step_on(const bnnhmc_model* model, const bnnhmc_launch* launch, 
   a.status = w.status;
   a.rank_hash = w.rank_hash;
   int wgs = 0;
-  set_grid(a, 1, G, &wgs);
+  set_grid(a, 1, G, plan.wide, &wgs);
   // status words and the exchange area start from zero on every call
   HIP_TRY(launch_fill_u32(w.status, STATUS_WORDS, 0u, st));
   HIP_TRY(clear_exchange(w, a, 1, plan.wide, st));
@@ -1032,8 +1052,10 @@ int bnnhmc_init_chains(bnnhmc_sampler* s, const float* w0) {
   HIP_TRY(launch_fill_u32((unsigned*)s->st_sel, C, 0u, s->stream));
   HIP_TRY(launch_fill_u32((unsigned*)s->st_nacc, C, 0u, s->stream));
   // bootstrap (main.h:191-202): log-posterior rows and gradient at the initial state
-  for (int base = 0; base < s->n_chains; base += s->plan.max_groups) {
-    const int groups = std::min(s->plan.max_groups, s->n_chains - base);
+  // (in the batches the transitions will run in: a chain's sums are then added in one order for its
+  // whole life)
+  for (int base = 0, groups = 0; base < s->n_chains; base += groups) {
+    groups = batch_size(s->plan, s->n_chains - base);
     KArgs a = base_args(s);
     a.mode = MODE_STEPS;
     a.L = 1;
@@ -1065,8 +1087,8 @@ int bnnhmc_run(bnnhmc_sampler* s, int n_transitions) {
   if (n_transitions == 0) return BNNHMC_OK;
   long launches = 0;
   HIP_TRY(hipEventRecord(s->ev0, s->stream));
-  for (int base = 0; base < s->n_chains; base += s->plan.max_groups) {
-    const int groups = std::min(s->plan.max_groups, s->n_chains - base);
+  for (int base = 0, groups = 0; base < s->n_chains; base += groups) {
+    groups = batch_size(s->plan, s->n_chains - base);
     for (int done = 0; done < n_transitions; done += s->plan.transitions_per_launch) {
       KArgs a = base_args(s);
       a.mode = MODE_TRANSITIONS;

@@ -295,16 +295,17 @@ def test_200_windows_are_batched_without_crosstalk(pkg, lib, orc):
     big.run(burn + keep)
     assert big.timing()["grad_evals"] == 200 * 2 * L
     checks = {}
-    for chain in (0, 63, 64, 191, 192, 199):
+    for chain in (0, 63, 64, 127, 128, 150, 191, 192, 199):
         checks[chain] = (big.get_samples(chain), big.get_traces(chain), big.get_chain_state(chain),
-                         big.get_window_data(chain) if chain in (0, 199) else None)
+                         big.get_window_data(chain) if chain in (0, 150, 199) else None)
         assert np.all(np.isfinite(checks[chain][0])) and checks[chain][2]["transitions_done"] == 2
         assert checks[chain][2]["n_accepted"] >= 1 and np.abs(checks[chain][0]).max() > 0
     big.close()
     assert not np.array_equal(checks[63][0], checks[64][0])       # different windows, different chains
-    # chain 0 sat in a batch of 64 at 4 workgroups per chain, chain 199 in the tail batch of 8 at 32:
-    # each must equal, bit for bit, a sampler that holds only that window and is launched that way
-    for chain, G in ((0, 4), (199, 32)):
+    # chain 0 sat in the batch of 128 at 2 workgroups per chain, chain 150 in the batch of 64 at 4, chain
+    # 199 in the tail batch of 8 at 32: each must equal, bit for bit, a sampler that holds only that
+    # window and is launched that way
+    for chain, G in ((0, 2), (150, 4), (199, 32)):
         X, y = checks[chain][3]
         h1 = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=eps0, seed=0,
                              adapt_steps=0, chain_id_base=chain)
