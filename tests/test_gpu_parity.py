@@ -236,11 +236,13 @@ def _run_pair(pkg, lib, orc, kind, n, L, burn, keep, eps0, G, layer="mfma", seed
 
 
 @pytest.mark.parametrize("layer,G,tpl", [("mfma", 8, 5), ("ffma", 8, 5), ("mfma", 128, 7), ("mfma", 0, 4),
-                                         ("ffma", 128, 60)])
+                                         ("ffma", 128, 60), ("mfma", 1, 5), ("mfma", 2, 9), ("mfma", 16, 5),
+                                         ("mfma", 32, 6), ("ffma", 32, 5)])
 def test_transitions_match_oracle_decisions(pkg, lib, orc, layer, G, tpl):
-    """G = 8: all workgroups read all records; G = 128 and G = 0 (one chain: widened to 256): the
-    two-phase exchange, in which the sum of the per-row log-likelihood differences travels through
-    the totals record; several launches per run (tpl transitions each)."""
+    """G up to 16: all workgroups read all records (1, 2 and 32 are what the automatic batches of a
+    200-window run use); G = 32, 128 and G = 0 (one chain: widened to 256): the exchange by slices, in
+    which the sum of the per-row log-likelihood differences travels through the totals record;
+    several launches per run (tpl transitions each)."""
     say("transitions layer=%s G=%d" % (layer, G))
     n, L, burn, keep = 2048, 20, 30, 30
     out, ref, (om, X, y) = _run_pair(pkg, lib, orc, "t_stiff", n, L, burn, keep, 0.01, G, layer=layer, tpl=tpl)
