@@ -44,6 +44,10 @@ struct MfmaWideLayer {
   float db1acc[NT];
   float db2acc;
   double dl;
+  // per step (prepare_step): the layer-2 sum starts from (sum of w2 - b2) sr2 -- high part in lane
+  // n = 0, low part in lane n = 1 of every row of 16 lanes -- and lane n = 2 adds y sr2; sr2 is the
+  // power of two next to 1 / scale, the factor (1 / scale) / sr2 is applied to the finished sum
+  float y_0, y_k, ratio, w2_scale;  // w2_scale = -2 sr2
 
   struct Tile {
     f4 xa[KQ];
@@ -61,6 +65,27 @@ struct MfmaWideLayer {
     }
     db2acc = 0.0f;
     dl = 0.0;
+  }
+
+  // The pointwise stage works with s = 1 / (1 + 2^t) = (1 + tanh x) / 2 and never forms h = 2 s - 1:
+  //   yhat = sum w2 h + b2 = 2 sum w2 s - (sum w2 - b2)        (the constant: once per step, in double)
+  //   dw2  = sum g h       = 2 sum g s - sum g                  (add_partials)
+  //   1 - h^2 = 4 (s - s^2)                                     (the 4 goes into add_partials)
+  // Scaling by a power of two keeps every product of the layer-2 sum exact.
+  __device__ __forceinline__ void prepare_step(const float* s_w, const ModelConsts& mc) {
+    const int lane = threadIdx.x & 63, n = lane & 15;
+    const uint32_t sr2_bits = (__builtin_bit_cast(uint32_t, mc.scale_recp) + 0x00400000u) & 0x7F800000u;
+    const float sr2 = __builtin_bit_cast(float, sr2_bits);
+    ratio = mc.scale_recp * __builtin_bit_cast(float, 0x7F000000u - sr2_bits);
+    double sum = 0.0;
+    for (int c = lane; c < D1; c += 64) sum += (double)s_w[oW2 + c];
+#pragma unroll
+    for (int msk = 1; msk < 64; msk <<= 1) sum += shfl_xor_d(sum, msk);
+    const double c0 = (sum - (double)s_w[oB2]) * (double)sr2;
+    const float c0_hi = (float)c0, c0_lo = (float)(c0 - (double)c0_hi);
+    y_0 = n == 0 ? c0_hi : (n == 1 ? c0_lo : 0.0f);
+    y_k = n == 2 ? sr2 : 0.0f;
+    w2_scale = -2.0f * sr2;
   }
 
   // rows past the end read as the last row (their gradient is masked to zero); any alignment
@@ -121,57 +146,66 @@ struct MfmaWideLayer {
       for (int t = 0; t < NT; ++t)
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bw[s & 1][t], acc[t], 0, 0, 0);
     }
-    // tanh(x) = 2 / (1 + 2^t) - 1 (kernel_helpers.h:34-42 without the small-|x| identity branch)
-    const float b2s = s_w[oB2] * mc.scale_recp;
-    float yh[4] = {0.f, 0.f, 0.f, 0.f};
+    // s = 1 / (1 + 2^t) (kernel_helpers.h:34-42 without the small-|x| identity branch, see prepare_step)
+    float yh[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) yh[j] = __builtin_fmaf(ti.yv[j], y_k, y_0);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      const float w2y = -s_w[oW2 + 16 * t + n] * mc.scale_recp;
+      const float w2y = s_w[oW2 + 16 * t + n] * w2_scale;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float e = __builtin_amdgcn_exp2f(acc[t][j]);
-        const float h = __builtin_fmaf(__builtin_amdgcn_rcpf(1.0f + e), 2.0f, -1.0f);
-        acc[t][j] = h;
-        yh[j] = __builtin_fmaf(w2y, h, yh[j]);
+        const float sg = __builtin_amdgcn_rcpf(1.0f + e);
+        acc[t][j] = sg;
+        yh[j] = __builtin_fmaf(w2y, sg, yh[j]);
       }
     }
-    float g[4];
-    float gsum = 0.0f;
+    // scaled residual (y - yhat - b2) / scale of the four rows 4 q + j (mcmc_step_ffma.h:293), in bank
+    // j of one register; the loss gradient is computed on that one register
+    const float dz = row16_reduce4(yh[0], yh[1], yh[2], yh[3]) * ratio;
+    float gz;
+    if (LIK == 0) gz = dz * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(dz, dz, mc.df));
+    else gz = dz * mc.scale_recp;
+    float g[4] = {row16_bcast<0>(gz), row16_bcast<1>(gz), row16_bcast<2>(gz), row16_bcast<3>(gz)};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      // scaled residual (y - yhat - b2) / scale, mcmc_step_ffma.h:293
-      const float diff = __builtin_fmaf(ti.yv[j], mc.scale_recp, row16_allreduce(yh[j]) - b2s);
-      float gj;
-      if (LIK == 0) gj = diff * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(diff, diff, mc.df));
-      else gj = diff * mc.scale_recp;
       const bool valid = FULL || (row0 + 4 * q + j < cx.n);
-      gj = valid ? gj : 0.0f;  // mcmc_step_ffma.h:301
-      g[j] = gj;
-      gsum += gj;
-      if (LAST) {
+      g[j] = valid ? g[j] : 0.0f;  // mcmc_step_ffma.h:301
+      db2acc += g[j];
+    }
+    if (LAST) {
+      const float d4[4] = {row16_bcast<0>(dz), row16_bcast<1>(dz), row16_bcast<2>(dz), row16_bcast<3>(dz)};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool valid = FULL || (row0 + 4 * q + j < cx.n);
         if (n == 0 && valid) {
           const int row = row0 + 4 * q + j;
-          const float lv = lik_value<LIK>(mc, diff);
+          const float lv = lik_value<LIK>(mc, d4[j]);
           const float prev = cx.ell_prev ? cx.ell_prev[row] : 0.0f;
           if (cx.ell_new) cx.ell_new[row] = lv;
           dl += (double)(lv - prev);
         }
       }
     }
-    db2acc += gsum;
-    // delta without its factor w2[c] (applied once per step to the sums)
+    // GEMM2 operands: u = s - s^2 stays where it is (A), g goes into the rows of x (B); the factors
+    // 4 w2[c] of delta are applied once per step to the sums
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      float s = 0.0f;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float h = acc[t][j];
-        dw2acc[t] = __builtin_fmaf(g[j], h, dw2acc[t]);
-        const float d = __builtin_fmaf(-h, h, 1.0f) * g[j];
-        acc[t][j] = d;
-        s += d;
+        const float sg = acc[t][j];
+        dw2acc[t] = __builtin_fmaf(g[j], sg, dw2acc[t]);
+        const float u = __builtin_fmaf(-sg, sg, sg);
+        acc[t][j] = u;
+        db1acc[t] = __builtin_fmaf(u, g[j], db1acc[t]);
       }
-      db1acc[t] += s;
+    }
+    f2 gx[4][FV];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int v = 0; v < FV; ++v) gx[j][v] = ti.xb[j][v] * g[j];
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -180,8 +214,8 @@ struct MfmaWideLayer {
 #pragma unroll
         for (int v = 0; v < FV; ++v) {
           dacc[t][2 * v] =
-              __builtin_amdgcn_mfma_f32_16x16x4f32(acc[t][j], ti.xb[j][v][0], dacc[t][2 * v], 0, 0, 0);
-          dacc[t][2 * v + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(acc[t][j], ti.xb[j][v][1],
+              __builtin_amdgcn_mfma_f32_16x16x4f32(acc[t][j], gx[j][v][0], dacc[t][2 * v], 0, 0, 0);
+          dacc[t][2 * v + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(acc[t][j], gx[j][v][1],
                                                                     dacc[t][2 * v + 1], 0, 0, 0);
         }
       }
@@ -256,7 +290,8 @@ struct MfmaWideLayer {
   }
 
   // add this wave's partial sums into the workgroup record in LDS (canonical parameter numbers);
-  // `first` overwrites.  The factor w2[c] left out of delta is applied here.
+  // `first` overwrites.  The factor 4 w2[c] left out of delta is applied here, and dw2 is put
+  // together from the sums of g s and of g (see prepare_step).
   __device__ __forceinline__ void add_partials(float* red, const float* s_w, bool first) {
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
 #pragma unroll
@@ -264,7 +299,7 @@ struct MfmaWideLayer {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int c = 16 * t + 4 * q + j;
-        const float w2c = s_w[oW2 + c];
+        const float w2c = 4.0f * s_w[oW2 + c];
 #pragma unroll
         for (int ft = 0; ft < FT; ++ft) {
           const int f = 32 * (ft >> 1) + 2 * n + (ft & 1);
@@ -274,14 +309,14 @@ struct MfmaWideLayer {
         }
       }
       // sums over the four row groups q in a fixed order
-      float vb = db1acc[t], vw = dw2acc[t];
+      float vb = db1acc[t], vw = 2.0f * dw2acc[t] - db2acc;
       vb += __shfl_xor(vb, 16);
       vb += __shfl_xor(vb, 32);
       vw += __shfl_xor(vw, 16);
       vw += __shfl_xor(vw, 32);
       if (q == 0) {
         const int c = 16 * t + n;
-        const float b = vb * s_w[oW2 + c];
+        const float b = vb * (4.0f * s_w[oW2 + c]);
         red[oB1 + c] = first ? b : red[oB1 + c] + b;
         red[oW2 + c] = first ? vw : red[oW2 + c] + vw;
       }
@@ -412,6 +447,7 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
       }
       __syncthreads();
       layer.zero_acc();
+      layer.prepare_step(s_w, mc);
       const bool last = s == a.L - 1;
       if (last) {
         cx.ell_prev = ell_cur;
