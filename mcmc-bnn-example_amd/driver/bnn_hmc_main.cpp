@@ -132,9 +132,11 @@ int main(int argc, char** argv) {
   int n_dev = 0, cus = 0;
   char arch[64];
   CHECK(bnnhmc_device_info(&n_dev, &cus, arch, sizeof(arch)));
-  std::printf("Device 0: %s, %d compute units. %d window(s) x %d chain(s), %d workgroups per chain, %s layer.\n",
-              arch, cus, o.windows, o.chains, launch.cus_per_chain,
-              o.layer == BNNHMC_LAYER_FFMA ? "FFMA" : "MFMA");
+  char groups[64];
+  if (launch.cus_per_chain > 0) std::snprintf(groups, sizeof(groups), "%d workgroups per chain", launch.cus_per_chain);
+  else std::snprintf(groups, sizeof(groups), "workgroups per chain chosen by the library");
+  std::printf("Device 0: %s, %d compute units. %d window(s) x %d chain(s), %s, %s layer.\n", arch, cus,
+              o.windows, o.chains, groups, o.layer == BNNHMC_LAYER_FFMA ? "FFMA" : "MFMA");
 
   bnnhmc_sampler* s = nullptr;
   CHECK(bnnhmc_create(&model, &hmc, &launch, o.windows, o.chains, &s));

@@ -91,7 +91,8 @@ def main(out):
                          "source": "rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over every trajectory-kernel "
                                    "dispatch of one bench.py run, each scaled by the same counter on a 1 GiB "
                                    "copy kernel",
-                         "cus_per_chain": d["config"]["cus_per_chain"] if d else None}},
+                         "launches_chains_x_workgroups_per_chain":
+                             d["config"].get("launches_chains_x_workgroups_per_chain") if d else None}},
                   open(os.path.join(out, "traffic.json"), "w"), indent=1)
     sq = find(os.path.join(out, "pmc_SQ"), "*counter_collection.csv")
     if sq:
