@@ -103,7 +103,7 @@ int bnnhmc_device_info(int* n_devices, int* compute_units, char* arch, size_t ar
  * (NULL = default stream).  Calls are asynchronous on `stream` unless stated.
  * ---------------------------------------------------------------------------------------------- */
 
-/* Device scratch the step operator needs (per-workgroup gradient partials and barrier words); the
+/* Device scratch the step operator needs (per-workgroup gradient records, status words); the
  * counterpart of the reference's grid_sync_workspace (include/mcmc/main.h:171,
  * include/mcmc/mcmc_step_tc.h:597-612).  The workspace must be 16-byte aligned (any hipMalloc
  * result is). */

@@ -126,16 +126,16 @@ struct KArgs {
   uint32_t seed;
   uint32_t rng_id_base;  // RNG key word 1 of chain c is rng_id_base + c
   // ---- cross-workgroup exchange ----
-  float* partials;     // [group][2][G][slot]
-  float* totals;       // [group][slot]: reduced gradient, two-phase reduction only
-  int two_phase;       // 1: each workgroup reduces a slice of the parameters, then all read the totals
-  unsigned* barrier;   // [group][BARRIER_STRIDE_WORDS]
+  float* partials;     // [group][2][G][slot]; 22 -> 40 -> 1: slots of 8-byte packets {value, step number}
+  float* totals;       // [group][slot]: reduced gradient, reduction by slices only
+  int two_phase;       // 1: the first workgroups each reduce a slice of the parameters, then all read the totals
+  unsigned* barrier;   // [group][BARRIER_STRIDE_WORDS], 64 -> 128 -> 1 only
   unsigned* status;    // [0] abort flag, [1] timed-out workgroup + 1; [4..9] belong to the hash check
   unsigned long long* rank_hash;  // [workgroup in group-major order]: hash of the state this workgroup
                                   // integrated; all workgroups of a chain group must agree
   unsigned spin_limit;
   float* wg_scratch;   // wide-layer kernel, MODE_TRANSITIONS: [workgroup][3][P_AL] accepted w, g and start momentum
-  int debug_drop_rank; // >= 0: this rank of every group never signals arrival (exercises the timeout path)
+  int debug_drop_rank; // >= 0: this rank of every group never publishes (exercises the timeout path)
   int debug_perturb_hash_rank;  // >= 0: this rank of every group flips a bit of its state hash
   unsigned* debug_xcc; // optional [workgroup] XCC id
   unsigned long long* debug_phase;  // optional [workgroup][10]: cycles per phase of a step, launch ticks

@@ -5,7 +5,8 @@
 // ("chain group"); every workgroup of the group redundantly integrates all P parameters, so only
 // the gradient crosses workgroups, once per leapfrog step, through a deterministic two-stage
 // reduction: (1) wavefront partials -> LDS slots -> fixed-order sum per workgroup, (2) per-workgroup
-// partials in global scratch -> group barrier -> fixed-order sum in every workgroup.
+// records of flagged packets in global scratch, polled by the readers (no barrier) -> fixed-order
+// sum in every workgroup, or, for wide groups, slice by slice in the first workgroups of the group.
 //
 // What it replaces in the reference: leapfrog_step_kernel (include/mcmc/mcmc_step_ffma.h:154-379),
 // the persistent mcmc_step_kernel with its grid barrier (include/mcmc/mcmc_step_tc.h:597-677),
