@@ -44,15 +44,16 @@ struct MfmaWideLayer {
   float db1acc[NT];
   float db2acc;
   double dl;
-  // per step (prepare_step): the layer-2 sum starts from (sum of w2 - b2) sr2 -- high part in lane
-  // n = 0, low part in lane n = 1 of every row of 16 lanes -- and lane n = 2 adds y sr2; sr2 is the
-  // power of two next to 1 / scale, the factor (1 / scale) / sr2 is applied to the finished sum
-  float y_0, y_k, ratio, w2_scale;  // w2_scale = -2 sr2
+  // per step (prepare_step): every lane's part of the layer-2 sum starts from its own share of the
+  // constant (sum of w2 - b2) sr2; what the roundings of the 16 shares leave over, and the target
+  // times sr2, are added to the finished row sum.  sr2 is the power of two next to 1 / scale, the factor
+  // (1 / scale) / sr2 is applied to the finished sum
+  float y_0, rho, sr2v, ratio, w2_scale;  // w2_scale = -2 sr2
 
   struct Tile {
     f4 xa[KQ];
     f2 xb[4][FV];
-    f4 yv;
+    float y1;  // target of row 4 q + (n >> 2): lane n sits in bank n >> 2, where that row's sum lands
   };
 
   __device__ __forceinline__ void zero_acc() {
@@ -77,14 +78,20 @@ struct MfmaWideLayer {
     const uint32_t sr2_bits = (__builtin_bit_cast(uint32_t, mc.scale_recp) + 0x00400000u) & 0x7F800000u;
     const float sr2 = __builtin_bit_cast(float, sr2_bits);
     ratio = mc.scale_recp * __builtin_bit_cast(float, 0x7F000000u - sr2_bits);
-    double sum = 0.0;
-    for (int c = lane; c < D1; c += 64) sum += (double)s_w[oW2 + c];
+    // the share of lane n: its hidden units 16 t + n [and b2 in lane 0]; a large constant in one lane
+    // would set the rounding grid of that lane's whole sum, and where hidden units saturate the terms
+    // take few distinct values, so roundings would repeat from row to row instead of averaging out
+    double share = 0.0;
 #pragma unroll
-    for (int msk = 1; msk < 64; msk <<= 1) sum += shfl_xor_d(sum, msk);
-    const double c0 = (sum - (double)s_w[oB2]) * (double)sr2;
-    const float c0_hi = (float)c0, c0_lo = (float)(c0 - (double)c0_hi);
-    y_0 = n == 0 ? c0_hi : (n == 1 ? c0_lo : 0.0f);
-    y_k = n == 2 ? sr2 : 0.0f;
+    for (int t = 0; t < NT; ++t) share += (double)s_w[oW2 + 16 * t + n];
+    if (n == 0) share -= (double)s_w[oB2];
+    share *= (double)sr2;
+    y_0 = (float)share;
+    double rest = share - (double)y_0;
+#pragma unroll
+    for (int msk = 1; msk < 16; msk <<= 1) rest += shfl_xor_d(rest, msk);
+    rho = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, (float)rest)));
+    sr2v = sr2;
     w2_scale = -2.0f * sr2;
   }
 
@@ -101,8 +108,8 @@ struct MfmaWideLayer {
       const float* rb = cx.X + (size_t)rowb * D0 + 2 * n;
 #pragma unroll
       for (int v = 0; v < FV; ++v) ti.xb[j][v] = f2{rb[32 * v], rb[32 * v + 1]};
-      ti.yv[j] = cx.y[rowb];
     }
+    ti.y1 = cx.y[min(row0 + 4 * q + (n >> 2), last)];
   }
 
   // wait until at most N memory operations are outstanding; the tile's registers are tied to the
@@ -113,7 +120,7 @@ struct MfmaWideLayer {
     asm volatile("s_waitcnt vmcnt(%[cnt])"
                  : "+v"(t.xa[0]), "+v"(t.xa[1]), "+v"(t.xa[2]), "+v"(t.xa[3]), "+v"(t.xb[0][0]),
                    "+v"(t.xb[0][1]), "+v"(t.xb[1][0]), "+v"(t.xb[1][1]), "+v"(t.xb[2][0]),
-                   "+v"(t.xb[2][1]), "+v"(t.xb[3][0]), "+v"(t.xb[3][1]), "+v"(t.yv)
+                   "+v"(t.xb[2][1]), "+v"(t.xb[3][0]), "+v"(t.xb[3][1]), "+v"(t.y1)
                  : [cnt] "n"(N)
                  : "memory");
   }
@@ -147,9 +154,7 @@ struct MfmaWideLayer {
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bw[s & 1][t], acc[t], 0, 0, 0);
     }
     // s = 1 / (1 + 2^t) (kernel_helpers.h:34-42 without the small-|x| identity branch, see prepare_step)
-    float yh[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) yh[j] = __builtin_fmaf(ti.yv[j], y_k, y_0);
+    float yh[4] = {y_0, y_0, y_0, y_0};
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const float w2y = s_w[oW2 + 16 * t + n] * w2_scale;
@@ -163,7 +168,7 @@ struct MfmaWideLayer {
     }
     // scaled residual (y - yhat - b2) / scale of the four rows 4 q + j (mcmc_step_ffma.h:293), in bank
     // j of one register; the loss gradient is computed on that one register
-    const float dz = row16_reduce4(yh[0], yh[1], yh[2], yh[3]) * ratio;
+    const float dz = (row16_reduce4(yh[0], yh[1], yh[2], yh[3]) + __builtin_fmaf(ti.y1, sr2v, rho)) * ratio;
     float gz;
     if (LIK == 0) gz = dz * mc.g_scale * __builtin_amdgcn_rcpf(__builtin_fmaf(dz, dz, mc.df));
     else gz = dz * mc.scale_recp;
@@ -240,7 +245,7 @@ struct MfmaWideLayer {
       static_assert(KQ == 4 && FV == 2, "operand list below is written for D0 = 64");
       const unsigned oa = (unsigned)((n * D0 + KS * q) * 4);
       const unsigned ob = (unsigned)(((4 * q) * D0 + 2 * n) * 4);
-      const unsigned oy = (unsigned)(4 * q * 4);
+      const unsigned oy = (unsigned)((4 * q + (n >> 2)) * 4);
       auto issue = [&](Tile& t, int tile) {
         tile = tile < fast_end ? tile : fast_end - 1;
         const float* bx = cx.X + (size_t)tile * (16 * D0);
@@ -259,11 +264,11 @@ struct MfmaWideLayer {
             "global_load_dwordx2 %[b21], %[ob], %[bx] offset:640\n\t"
             "global_load_dwordx2 %[b30], %[ob], %[bx] offset:768\n\t"
             "global_load_dwordx2 %[b31], %[ob], %[bx] offset:896\n\t"
-            "global_load_dwordx4 %[yv], %[oy], %[by]"
+            "global_load_dword %[yv], %[oy], %[by]"
             : [a0] "=&v"(t.xa[0]), [a1] "=&v"(t.xa[1]), [a2] "=&v"(t.xa[2]), [a3] "=&v"(t.xa[3]),
               [b00] "=&v"(t.xb[0][0]), [b01] "=&v"(t.xb[0][1]), [b10] "=&v"(t.xb[1][0]),
               [b11] "=&v"(t.xb[1][1]), [b20] "=&v"(t.xb[2][0]), [b21] "=&v"(t.xb[2][1]),
-              [b30] "=&v"(t.xb[3][0]), [b31] "=&v"(t.xb[3][1]), [yv] "=&v"(t.yv)
+              [b30] "=&v"(t.xb[3][0]), [b31] "=&v"(t.xb[3][1]), [yv] "=&v"(t.y1)
             : [oa] "v"(oa), [ob] "v"(ob), [oy] "v"(oy), [bx] "s"(bx), [by] "s"(by)
             : "memory");
       };

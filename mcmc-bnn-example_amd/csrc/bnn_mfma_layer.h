@@ -74,9 +74,9 @@ struct MfmaLayer {
                        // keeps the coefficients exact: the dot cancels from terms of size |w2| k to a
                        // residual thousands of times smaller, and a rounding error in a coefficient
                        // would be the same in every row and add up over the rows instead of averaging out
-  float y_k[4];        // y_k[j]: k2 in lane n == j, else 0 (lane n < 4 holds the target of row 4 q + n)
-  float y_0;           // the constant part of the dot, (sum_c w2[c] - b2) k2, computed in double and
-                       // split over lanes n == 4 (leading part) and n == 5 (remainder)
+  float k2v;           // k2 (the same in every lane): the target y enters as y k2 after the row sums
+  float y_0;           // where this lane's partial sum starts: its share of the constant (sum_c w2[c] - b2) k2
+  float rho;           // what the roundings of the 16 shares leave over (the same in every lane)
   float ratio;         // k / k2 (exact)
   // sums over rows of s (1 - s) g' x_aug, g' = g k2 / k (Gaussian) or g (Student-t):
   f4 dacc_e[NT];       //   features 0 .. 15
@@ -92,7 +92,7 @@ struct MfmaLayer {
     f2 xa[KP];   // GEMM1 operand
     float xe[4]; // GEMM2e operand: feature n of rows 4 q + j
     f2 xf[4];    // GEMM2f operand: features 16 + 2 jj, 17 + 2 jj of rows 4 q + j
-    float y1;    // target of row 4 q + (n & 3)
+    float y1;    // target of row 4 q + (n >> 2): lane n sits in bank n >> 2, where that row's sum lands
   };
 
   static constexpr float kExp2Scale = -2.88539008177792681472f;  // -2 / ln 2, kernel_helpers.h:37
@@ -106,7 +106,7 @@ struct MfmaLayer {
     const float k2 = __builtin_bit_cast(float, k2_bits);
     ratio = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
         int, k * __builtin_bit_cast(float, 0x7F000000u - k2_bits))));
-    double w2sum = 0.0;
+    double w2lane = 0.0;  // sum of the layer-2 weights of this lane's hidden units
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int c = 16 * t + n;
@@ -121,17 +121,22 @@ struct MfmaLayer {
         w1b[s][t] = cv ? v * kExp2Scale : 0.0f;
       }
       const float w2c = cv ? s_w[oW2 + cc] : 0.0f;
-      w2sum += (double)w2c;
+      w2lane += (double)w2c;
       w2g[t] = -2.0f * w2c * k2;
     }
-    // sum over all hidden units in double, the same bits in every lane of a row of 16
+    // Each lane's partial sum starts from its own share of the constant, k2 (sum of its w2 [- b2 in
+    // lane 0]), so that it stays of the size of k2 sum w2 h (the tanh form's): a large constant in one
+    // lane would set the rounding grid of that lane's whole sum, and where hidden units saturate (s
+    // exactly 0 or 1) the terms take few distinct values, so roundings repeat from row to row instead of
+    // averaging out.  What the 16 roundings of the shares leave over (exactly known in double) is
+    // added after the row sum, together with the target.
+    const double share = (w2lane - (n == 0 ? (double)s_w[oB2] : 0.0)) * (double)k2;
+    y_0 = (float)share;
+    double rest = share - (double)y_0;
 #pragma unroll
-    for (int msk = 1; msk < 16; msk <<= 1) w2sum += shfl_xor_d(w2sum, msk);
-    const double c0 = (w2sum - (double)s_w[oB2]) * (double)k2;
-    const float c0_hi = (float)c0, c0_lo = (float)(c0 - (double)c0_hi);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) y_k[j] = n == j ? k2 : 0.0f;
-    y_0 = n == 4 ? c0_hi : (n == 5 ? c0_lo : 0.0f);
+    for (int msk = 1; msk < 16; msk <<= 1) rest += shfl_xor_d(rest, msk);
+    rho = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, (float)rest)));
+    k2v = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, k2)));
   }
 
   __device__ __forceinline__ void zero_acc() {
@@ -173,7 +178,7 @@ struct MfmaLayer {
       ti.xe[j] = rb[n];
       ti.xf[j] = f0 < D0 ? f2{rb[fc], rb[fc + 1]} : const_f(jj);
     }
-    ti.y1 = cx.y[min(row0 + 4 * q + jj, last)];
+    ti.y1 = cx.y[min(row0 + 4 * q + (n >> 2), last)];
   }
 
   // ordinary loads of a full, aligned tile through per-lane pointers (the plain and the software-
@@ -186,7 +191,7 @@ struct MfmaLayer {
     const float* pe;        // rows 4 q + j, feature n
     const float* pf0;       // rows 4 q + j, features 16 + 2 jj ..: real data or constants
     unsigned sf;
-    const float* py;        // row 4 q + jj
+    const float* py;        // row 4 q + (n >> 2)
     int tb;
   };
   __device__ __forceinline__ PlainPtrs plain_ptrs(const StepCtx& cx, int tb, int n, int q) const {
@@ -204,7 +209,7 @@ struct MfmaLayer {
     p.pf0 = f_const ? (16 + 2 * jj == D0 ? aug->one : aug->zero)
                     : cx.X + ((size_t)tb * 16 + 4 * q) * D0 + 16 + 2 * jj;
     p.sf = f_const ? 0u : (unsigned)tile_floats;
-    p.py = cx.y + 4 * q + jj;
+    p.py = cx.y + 4 * q + (n >> 2);
     return p;
   }
   __device__ __forceinline__ void load_plain(TileIn& ti, const PlainPtrs& p, int tile) const {
@@ -252,9 +257,7 @@ struct MfmaLayer {
   __device__ __forceinline__ void pointwise(f4 (&acc)[NT], const TileIn& ti, float (&ge)[4], f2 (&gf)[4],
                                             const StepCtx& cx, const ModelConsts& mc, int row0, int n,
                                             int q) {
-    float yh[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) yh[j] = __builtin_fmaf(ti.y1, y_k[j], y_0);
+    float yh[4] = {y_0, y_0, y_0, y_0};
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -268,7 +271,7 @@ struct MfmaLayer {
     // (y - yhat - b2) k2 of the four rows 4 q + j, in bank j of one register; the loss gradient
     // (Gaussian: that value itself, its factor k / k2 is applied to the sums once per step;
     // Student-t: mcmc_step_ffma.h:293-301) is computed on that one register
-    const float rz = row16_reduce4(yh[0], yh[1], yh[2], yh[3]);
+    const float rz = row16_reduce4(yh[0], yh[1], yh[2], yh[3]) + __builtin_fmaf(ti.y1, k2v, rho);
     float gz = rz, dz = rz;
     if (LIK == 0) {
       dz = rz * ratio;
@@ -501,7 +504,7 @@ struct MfmaLayer {
     lp.ol = lp.oa + 2 * (KP - 1) * 4;
     lp.oe = (unsigned)(((4 * q) * D0 + n) * 4);
     lp.of = (unsigned)(((4 * q) * D0 + 16 + 2 * lp.jj) * 4);
-    lp.oy = (unsigned)((4 * q + lp.jj) * 4);
+    lp.oy = (unsigned)((4 * q + (n >> 2)) * 4);
     const bool a_const = KS * q + 2 * (KP - 1) >= D0;
     const bool f_const = 16 + 2 * lp.jj >= D0;
     lp.mask_a = __builtin_amdgcn_ballot_w64(!a_const);
