@@ -6,9 +6,9 @@
 // one 16-row tile that way, checks the sums against a double-precision reference, and times the tile with
 // two waves per SIMD as in the production kernel: once with the operands fetched from LDS every tile (one
 // stage ahead of their use), once with the operands held in registers (what the arithmetic alone costs).
-// Result on MI355X: see profiles/tile_4x4_probe_mfma_22x40.txt -- no gain over the production tile, because
-// the bias gradients and the row-group bookkeeping that ride on the matrix instructions there become
-// vector instructions here, and the LDS fetches take issue slots.
+// Result on MI355X: no gain over the production tile -- the bias gradients and the row-group bookkeeping
+// that ride on the matrix instructions there become vector instructions here, the LDS fetches take issue
+// slots, and the chip clocks lower under this load.
 //
 //   tile_4x4_probe [tiles per wave]      (default 30000)
 //
@@ -56,7 +56,7 @@ struct Acc {
 
 template <bool FROM_LDS>
 __global__ __launch_bounds__(512) void probe(const float* Xg, const float* yg, const float* wg, float* out,
-                                             float* out_g, int tiles) {
+                                             float* out_g, int tiles, unsigned long long* clocks) {
   __shared__ float s_x[8][16 * D0 + 8];
   __shared__ float s_y[8][16];
   __shared__ float s_w[P + 3];
@@ -134,6 +134,7 @@ __global__ __launch_bounds__(512) void probe(const float* Xg, const float* yg, c
     yv_ = s_y[wave][4 * rg + q];
   };
   load_a(xa, xa5);
+  const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
   for (int it = 0; it < tiles; ++it) {
     asm volatile("" ::: "memory");
     // ---- GEMM1 (operands were read from LDS during the previous tile's GEMM2) ----
@@ -248,6 +249,10 @@ __global__ __launch_bounds__(512) void probe(const float* Xg, const float* yg, c
     for (int p = 0; p < 11; ++p) xa5[p] = xa5_n[p];
   }
 
+  if (threadIdx.x == 0 && blockIdx.x == 0 && clocks) {  // shader-clock ticks and 100 MHz ticks of one wave's loop
+    clocks[0] = __builtin_readcyclecounter() - c0;
+    clocks[1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
   // ---- results of wave 0 of block 0 (sums over the tile's 16 rows): canonical gradient without the prior ----
   if (blockIdx.x == 0 && wave == 0) {
     // dW1: dT[T][fg][i]: hidden 16 T + 4 q + i, feature 4 fg + jj, partial over rg: add the four rg (lanes n >> 2)
@@ -354,7 +359,7 @@ int main(int argc, char** argv) {
   HIP_CHECK(hipMemcpy(dy, y.data(), 64, hipMemcpyHostToDevice));
   HIP_CHECK(hipMemcpy(dw, w.data(), P * 4, hipMemcpyHostToDevice));
   HIP_CHECK(hipMemset(dout, 0, P * 4));
-  hipLaunchKernelGGL(probe<true>, dim3(1), dim3(512), 0, 0, dX, dy, dw, dout, dg, 1);
+  hipLaunchKernelGGL(probe<true>, dim3(1), dim3(512), 0, 0, dX, dy, dw, dout, dg, 1, (unsigned long long*)nullptr);
   HIP_CHECK(hipDeviceSynchronize());
   std::vector<float> got(P), gg(16);
   HIP_CHECK(hipMemcpy(got.data(), dout, P * 4, hipMemcpyDeviceToHost));
@@ -368,14 +373,17 @@ int main(int argc, char** argv) {
   for (int r = 0; r < 16; ++r) errg = std::fmax(errg, std::fabs(gg[r] - grow[r]));
   std::printf("one tile: max |grad - ref| = %.3e (scale %.3e) at parameter %d (got %.6f ref %.6f); max |g - ref| = %.3e\n",
               err, scale, worst, got[worst], gref[worst], errg);
-  // timing: 256 workgroups x 8 waves (two per SIMD)
+  // timing: 256 workgroups x 8 waves (two per SIMD); the shader clock is the ratio of the two counters one
+  // wave read around its loop
+  unsigned long long* dclk;
+  HIP_CHECK(hipMalloc(&dclk, 16));
   hipEvent_t e0, e1;
   HIP_CHECK(hipEventCreate(&e0));
   HIP_CHECK(hipEventCreate(&e1));
   for (int from_lds = 1; from_lds >= 0; --from_lds) {
     auto launch = [&](int t) {
-      if (from_lds) hipLaunchKernelGGL(probe<true>, dim3(256), dim3(512), 0, 0, dX, dy, dw, dout, dg, t);
-      else hipLaunchKernelGGL(probe<false>, dim3(256), dim3(512), 0, 0, dX, dy, dw, dout, dg, t);
+      if (from_lds) hipLaunchKernelGGL(probe<true>, dim3(256), dim3(512), 0, 0, dX, dy, dw, dout, dg, t, dclk);
+      else hipLaunchKernelGGL(probe<false>, dim3(256), dim3(512), 0, 0, dX, dy, dw, dout, dg, t, dclk);
     };
     launch(10 * tiles);  // warm-up long enough for the clocks to settle
     HIP_CHECK(hipDeviceSynchronize());
@@ -385,9 +393,12 @@ int main(int argc, char** argv) {
     HIP_CHECK(hipEventSynchronize(e1));
     float ms = 0;
     HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
-    std::printf("%-46s %d tiles per wave, two waves per SIMD: %.3f ms -> %.1f cycles per tile and SIMD at 2.37 GHz\n",
-                from_lds ? "operands fetched from LDS every tile:" : "operands held in registers:", tiles, ms,
-                ms * 1e-3 * 2.37e9 / (2.0 * tiles));
+    unsigned long long clk[2];
+    HIP_CHECK(hipMemcpy(clk, dclk, 16, hipMemcpyDeviceToHost));
+    const double mhz = (double)clk[0] / ((double)clk[1] * 1e-2);
+    std::printf("%-40s %d tiles per wave, two waves per SIMD: %.3f ms, shader clock %.0f MHz -> %.1f cycles per tile and SIMD\n",
+                from_lds ? "operands fetched from LDS every tile:" : "operands held in registers:", tiles, ms, mhz,
+                ms * 1e-3 * mhz * 1e6 / (2.0 * tiles));
   }
   return 0;
 }
