@@ -85,6 +85,9 @@ def main(out):
     if total_bytes and evals:
         lines.append("HBM traffic: %.4g bytes over %.0f gradient evaluations = %.0f bytes per evaluation" % (
             total_bytes, evals, total_bytes / evals))
+        if d:
+            lines.append("  = %.2f TB/s at the %.0f evaluations/s of the traced run (HBM peak 8 TB/s)" % (
+                total_bytes / evals * d["value"] / 1e12, d["value"]))
         key = "hmc_kernel_wide_64x128" if d and "64->128" in d["config"]["workload"] else (
             "hmc_kernel_%s_22x40" % (d["config"]["layer"] if d else "mfma"))
         json.dump({key: {"bytes_per_grad_eval": total_bytes / evals,
