@@ -1,5 +1,6 @@
-// The MFMA layer of the 22 -> 40 -> 1 trajectory kernel: both contractions of a 16-row tile on
-// v_mfma_f32_16x16x4_f32, the pointwise stage between them, and the tile loops.  In a header of its own
+// The MFMA layer of the 22 -> 40 -> 1 trajectory kernel: both contractions of a 16-row tile on the FP32
+// matrix instructions (16x16x4 tiles and 4x4x1 blocks), the pointwise stage between them, the tile loops
+// and the wave's partial sums.  In a header of its own
 // so that the tile-ceiling probe (tile_ceiling.hip) times exactly the code the kernel runs.
 #pragma once
 
