@@ -6,8 +6,9 @@ of the 22->40->1 Bayesian MLP, full batch of 58368 rows each (features ~ N(0,1),
 N(0, 0.01^2) noise, Gaussian likelihood, Gaussian weight prior), one chain per window, HMC with 1000
 leapfrog steps per transition, all 200 windows resident in HBM (1.07 GB).  A "step" is one HMC transition
 (momentum resampling, 1000 fused leapfrog gradient evaluations, log accept ratio, Metropolis decision,
-sample store) of every one of the 200 windows: the library runs them as batches of 128 chains at 2
-workgroups per chain, 64 chains at 4 and 8 chains at 32, each over all 256 compute units.  The warm-up transitions
+sample store) of every one of the 200 windows: the chains take turns, five transitions at a time, on
+launches of 128 chains at 2 workgroups per chain; what does not fill such a launch runs as 64 chains at 4,
+32 at 8, ... workgroups per chain, always over all 256 compute units.  The warm-up transitions
 are the burn-in (nothing stored), the timed ones store their samples.  The metric is leapfrog gradient
 evaluations per second; the minutes for 200 windows x (100 burn-in + 800 samples) are 900 steps plus the
 bootstrap evaluation, and --full runs that whole job.
@@ -233,7 +234,13 @@ def main():
                             4 if wide else 2, n_windows, cpw, min(n_chains, resident), d0, d1, n_rows, d0,
                             args.leapfrog),
             "layer": args.layer, "wgs_per_cu": wgs_per_cu,
-            "launches_chains_x_workgroups_per_chain": ", ".join("%d x %d" % bg for bg in plan),
+            "launches_chains_x_workgroups_per_chain": (
+                "%d x %d, the %d chains taking turns in quanta of %d transitions; what does not fill a launch runs "
+                "in the largest batches that fit (%s)" % (
+                    plan[0][0], plan[0][1], n_chains, args.transitions_per_launch,
+                    ", ".join("%d x %d" % bg for bg in plan[1:]))
+                if not wide and not launch.cus_per_chain and len(plan) > 1
+                else ", ".join("%d x %d" % bg for bg in plan)),
             "workgroups_last_launch": tm1["workgroups"], "compute_units": cus,
             "transitions_per_launch": args.transitions_per_launch,
             "eps0": float(hmc.eps0), "adapt_steps": int(hmc.adapt_steps),

@@ -1087,42 +1087,76 @@ int bnnhmc_run(bnnhmc_sampler* s, int n_transitions) {
   if (n_transitions == 0) return BNNHMC_OK;
   long launches = 0;
   HIP_TRY(hipEventRecord(s->ev0, s->stream));
-  for (int base = 0, groups = 0; base < s->n_chains; base += groups) {
-    groups = batch_size(s->plan, s->n_chains - base);
-    for (int done = 0; done < n_transitions; done += s->plan.transitions_per_launch) {
-      KArgs a = base_args(s);
-      a.mode = MODE_TRANSITIONS;
-      a.n_trans = std::min(s->plan.transitions_per_launch, n_transitions - done);
-      a.chain_base = base;
-      a.st_w = s->st_w;
-      a.st_g = s->st_g;
-      a.st_stride = s->st_stride;
-      a.st_eps = s->st_eps;
-      a.st_t = s->st_t;
-      a.st_sel = s->st_sel;
-      a.st_nacc = s->st_nacc;
-      a.ell0 = s->ell0;
-      a.ell1 = s->ell1;
-      a.ell_stride = s->n_pad;
-      a.samples = s->samples;
-      a.n_samples = s->hmc.n_samples;
-      a.burn_in = s->hmc.burn_in;
-      a.adapt_steps = s->hmc.adapt_steps;
-      a.dec_adj = -s->hmc.decrement / (1.0f + s->hmc.decrement);
-      a.inc_adj = s->hmc.increment;
-      a.log_target = (float)std::log((double)s->hmc.target_rate);
-      a.tr_log_acpt = s->tr_la;
-      a.tr_accept = s->tr_acc;
-      a.tr_eps = s->tr_eps;
-      a.trace_len = s->trace_len;
-      a.seed = s->hmc.seed;
-      a.rng_id_base = s->hmc.chain_id_base;
-      a.debug_phase = s->debug_phase;
-      int rc = launch_and_count(s, a, groups);
+  auto launch = [&](int base, int groups, int n_trans) -> int {
+    KArgs a = base_args(s);
+    a.mode = MODE_TRANSITIONS;
+    a.n_trans = n_trans;
+    a.chain_base = base;
+    a.chain_wrap = s->n_chains;
+    a.st_w = s->st_w;
+    a.st_g = s->st_g;
+    a.st_stride = s->st_stride;
+    a.st_eps = s->st_eps;
+    a.st_t = s->st_t;
+    a.st_sel = s->st_sel;
+    a.st_nacc = s->st_nacc;
+    a.ell0 = s->ell0;
+    a.ell1 = s->ell1;
+    a.ell_stride = s->n_pad;
+    a.samples = s->samples;
+    a.n_samples = s->hmc.n_samples;
+    a.burn_in = s->hmc.burn_in;
+    a.adapt_steps = s->hmc.adapt_steps;
+    a.dec_adj = -s->hmc.decrement / (1.0f + s->hmc.decrement);
+    a.inc_adj = s->hmc.increment;
+    a.log_target = (float)std::log((double)s->hmc.target_rate);
+    a.tr_log_acpt = s->tr_la;
+    a.tr_accept = s->tr_acc;
+    a.tr_eps = s->tr_eps;
+    a.trace_len = s->trace_len;
+    a.seed = s->hmc.seed;
+    a.rng_id_base = s->hmc.chain_id_base;
+    a.debug_phase = s->debug_phase;
+    const int rc = launch_and_count(s, a, groups);
+    if (rc == BNNHMC_OK) ++launches;
+    return rc;
+  };
+  // every chain of [base, base + count) (indices wrap at n_chains) runs n_trans transitions, in the
+  // largest batches that fit
+  auto run_range = [&](int base, int count, int n_trans) -> int {
+    for (int groups = 0; count > 0; count -= groups, base = (base + groups) % s->n_chains) {
+      groups = batch_size(s->plan, count);
+      const int rc = launch(base, groups, n_trans);
       if (rc) return rc;
-      ++launches;
+    }
+    return BNNHMC_OK;
+  };
+  const int tpl = s->plan.transitions_per_launch;
+  const int full_batch = batch_size(s->plan, s->n_chains);
+  int rc0 = BNNHMC_OK;
+  if (s->plan.widen && !s->plan.wide && s->n_chains > full_batch) {
+    // More chains than fit at once: they take turns.  A chain's run is cut into quanta of tpl transitions;
+    // the quanta of all chains, in the order (pass, chain), are dealt to launches of full_batch chains
+    // each, so that every launch but the last few fills the device with its widest batch (a fixed split
+    // into batches would leave the last, small batch to run alone on wide, less efficient groups for the
+    // whole call).  A launch never holds two quanta of one chain (full_batch < n_chains), and a chain's
+    // quanta run in launch order.  What is left -- fewer than full_batch quanta, then the n mod tpl
+    // transitions every chain still owes -- runs in the largest batches that fit.
+    const long quanta = (long)s->n_chains * (n_transitions / tpl);
+    long dealt = 0;
+    for (; rc0 == BNNHMC_OK && quanta - dealt >= full_batch; dealt += full_batch)
+      rc0 = launch((int)(dealt % s->n_chains), full_batch, tpl);
+    if (rc0 == BNNHMC_OK && quanta > dealt)
+      rc0 = run_range((int)(dealt % s->n_chains), (int)(quanta - dealt), tpl);
+    if (rc0 == BNNHMC_OK && n_transitions % tpl) rc0 = run_range(0, s->n_chains, n_transitions % tpl);
+  } else {
+    for (int base = 0, groups = 0; rc0 == BNNHMC_OK && base < s->n_chains; base += groups) {
+      groups = batch_size(s->plan, s->n_chains - base);
+      for (int done = 0; rc0 == BNNHMC_OK && done < n_transitions; done += tpl)
+        rc0 = launch(base, groups, std::min(tpl, n_transitions - done));
     }
   }
+  if (rc0) return rc0;
   HIP_TRY(hipEventRecord(s->ev1, s->stream));
   int rc = check_status(s);
   if (rc) return rc;

@@ -79,6 +79,7 @@ struct KArgs {
   int G;            // workgroups per chain group
   int n_groups;     // chain groups in this launch
   int chain_base;   // global chain index of group 0
+  int chain_wrap;   // > 0: chain indices wrap around at this count (group g runs chain (chain_base + g) mod it)
   int chains_per_window;
   int fixed_window; // >= 0: every group reads this window
   int xcd_map;      // 1: blockIdx is spread round-robin over 8 XCDs, keep a group inside one XCD

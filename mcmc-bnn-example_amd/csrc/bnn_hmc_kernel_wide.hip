@@ -364,7 +364,8 @@ __global__ __launch_bounds__(T) void hmc_kernel_wide(const KArgs a) {
   }
   const int group = lin / a.G, rank = lin - group * a.G;
   if (group >= a.n_groups) return;
-  const int chain = a.chain_base + group;
+  int chain = a.chain_base + group;
+  if (a.chain_wrap > 0 && chain >= a.chain_wrap) chain -= a.chain_wrap;
   const int window = a.fixed_window >= 0 ? a.fixed_window : chain / a.chains_per_window;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
