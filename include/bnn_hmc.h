@@ -72,10 +72,12 @@ typedef struct bnnhmc_hmc {
 typedef struct bnnhmc_launch {
   int layer;          /* BNNHMC_LAYER_MFMA (v_mfma_f32_16x16x4_f32) or BNNHMC_LAYER_FFMA          */
   int cus_per_chain;  /* workgroups that share one chain's rows; 0 = automatic.  Sampler,         */
-                      /* 22 -> 40 -> 1: batches of the largest power-of-two number of chains that  */
-                      /* is left and fits, each over the whole device (200 chains on 256 CUs: 128   */
-                      /* chains x 2 workgroups, 64 x 4, 8 x 32; one chain: 256); 64 -> 128 -> 1: 4, */
-                      /* a smaller last batch widened.  Step operator: 256                          */
+                      /* 22 -> 40 -> 1: a batch is the largest power-of-two number of chains that */
+                      /* fits, spread over the whole device (one chain: 256 workgroups; 128 or     */
+                      /* more chains on 256 CUs: 2 each); more chains than fit take turns on such  */
+                      /* batches, transitions_per_launch transitions at a time, and what does not  */
+                      /* fill a batch runs in smaller, wider ones.  64 -> 128 -> 1: 4, a smaller    */
+                      /* last batch widened.  Step operator: 256                                    */
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */
   int threads;        /* threads per workgroup; default 512 for MFMA (every tile loop), 256 for  */
                       /* FFMA and with wgs_per_cu = 2.  The plain MFMA loop is also built for    */

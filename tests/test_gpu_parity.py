@@ -274,6 +274,42 @@ def test_transitions_match_oracle_decisions(pkg, lib, orc, layer, G, tpl):
     assert out["timing"]["grad_evals"] == T * L
 
 
+def test_more_chains_than_fit_take_turns(pkg, lib, orc):
+    """130 windows on a device that holds 128 chains at once: the chains take turns, 5 transitions at a
+    time, on launches of 128 (two of them here), what does not fill a launch runs in smaller batches
+    (the 4 quanta left over, then the 2 transitions every chain still owes).  Every chain must come out
+    with exactly 12 transitions, its own RNG stream and its own window: decisions, step sizes and samples
+    of chains from every part of that schedule against the oracle."""
+    n, L, burn, keep, n_windows, seed = 512, 6, 4, 8, 130, 77
+    model, om, gen = models(pkg, lib, "t_stiff", n)
+    hmc = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=0.01, seed=seed)
+    s = lib.create(model, hmc, lib.default_launch(transitions_per_launch=5), n_windows, 1)
+    for w in range(n_windows):
+        s.generate_window(w, **gen)
+    s.init_chains(None)
+    s.run(burn + keep)
+    assert s.timing()["grad_evals"] == n_windows * (burn + keep) * L
+    T = burn + keep
+    for chain in range(n_windows):
+        assert s.get_chain_state(chain)["transitions_done"] == T, chain
+    n_rejects = 0
+    for chain in (0, 1, 3, 4, 64, 125, 126, 127, 128, 129):
+        X, y = s.get_window_data(chain)
+        ref = orc.run_chain(om, ob.Hmc(L, burn, keep, burn, 0.01, 0.2, 0.1, 0.01, seed, chain), X, y)
+        tr, st = s.get_traces(chain), s.get_chain_state(chain)
+        margin = np.abs(np.array([orc.log_uniform(seed, chain, t) for t in range(T)]) - ref["log_acpt"])
+        clear = margin > 1e-3
+        assert np.array_equal(tr["accept"][clear], ref["accept"][clear]), chain
+        if clear.all():
+            assert tr["eps"].tobytes() == ref["eps"].tobytes(), chain
+            assert st["n_accepted"] == ref["n_accept"], chain
+            np.testing.assert_allclose(s.get_samples(chain), ref["samples"], rtol=0,
+                                       atol=2e-4 * max(1.0, float(np.abs(ref["samples"]).max())))
+        n_rejects += int(T - ref["n_accept"])
+    assert n_rejects > 0, "the inputs never reject: the decisions say nothing"
+    s.close()
+
+
 def test_divergent_trajectories_reject_and_restore(pkg, lib, orc):
     # the benchmark's stiff Gaussian posterior with the reference's eps0 = 0.01 diverges to inf/NaN
     # until adaptation has shrunk eps: every such transition must reject and leave the state alone
