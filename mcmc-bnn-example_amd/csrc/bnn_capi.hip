@@ -1052,8 +1052,8 @@ int bnnhmc_init_chains(bnnhmc_sampler* s, const float* w0) {
   HIP_TRY(launch_fill_u32((unsigned*)s->st_sel, C, 0u, s->stream));
   HIP_TRY(launch_fill_u32((unsigned*)s->st_nacc, C, 0u, s->stream));
   // bootstrap (main.h:191-202): log-posterior rows and gradient at the initial state
-  // (in the batches the transitions will run in: a chain's sums are then added in one order for its
-  // whole life)
+  // (in the batches the transitions run in when all chains fit at once: a chain's sums are then added
+  // in one order for its whole life)
   for (int base = 0, groups = 0; base < s->n_chains; base += groups) {
     groups = batch_size(s->plan, s->n_chains - base);
     KArgs a = base_args(s);

@@ -8,7 +8,7 @@ set -e
 ROOT="$(cd "$(dirname "$0")/.." && pwd)"
 OUT="$ROOT/gpurun_out/${PROFILE_DIR:-profile}"
 mkdir -p "$OUT"
-BENCH_ARGS="--steps 10 --warmup 5 --cpu-seconds 0 $*"
+BENCH_ARGS="--cpu-seconds 0 $*"
 cd /tmp && export TMPDIR=/tmp
 echo "== kernel trace + stats"
 timeout -s KILL 300 rocprofv3 --kernel-trace --stats -d "$OUT/trace" -o trace --output-format csv -- \

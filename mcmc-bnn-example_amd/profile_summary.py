@@ -52,6 +52,11 @@ def main(out):
         if trans:
             lines.append("average over the %d launches of transitions: %.3f ms" % (
                 len(trans), sum(trans) / len(trans)))
+        dt = bench_json(os.path.join(out, "bench_trace.json"))
+        if dt and 0 < dt["roofline"]["launches"] <= len(trans):
+            timed = trans[-dt["roofline"]["launches"]:]
+            lines.append("average over the last %d of them (the timed region of bench.py; the ones before are its "
+                         "warm-up): %.3f ms" % (len(timed), sum(timed) / len(timed)))
     d = bench_json(os.path.join(out, "bench_trace.json"))
     if d:
         lines.append("bench.py under the tracer: %.0f grad-evals/s, roofline frac %.3f, %.3f ms per launch "
