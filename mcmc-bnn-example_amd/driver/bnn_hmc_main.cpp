@@ -162,7 +162,9 @@ int main(int argc, char** argv) {
   CHECK(bnnhmc_init_chains(s, nullptr));
 
   // ------------------------------------------------------------------ run (main.h:204-287)
-  const int total = hmc.burn_in + hmc.n_samples, every = 10;
+  // calls of whole launch quanta, long enough that chains which take turns on the device (more windows
+  // than fit at once) do so on full launches
+  const int total = hmc.burn_in + hmc.n_samples, every = 5 * launch.transitions_per_launch;
   for (int done = 0; done < total; done += every) {
     CHECK(bnnhmc_run(s, std::min(every, total - done)));
     std::printf(".");
