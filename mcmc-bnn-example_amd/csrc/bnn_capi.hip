@@ -249,12 +249,19 @@ size_t exchange_slot_floats(int P, bool wide) {
   return (size_t)partial_slot_floats(P) * (wide ? 1 : 2);
 }
 
+// Totals records: one per chain group; a 22 -> 40 -> 1 group that reduces by slices (32 workgroups or
+// more, so at most wgs / 32 such groups at once) has TOTALS_COPIES of them.
+size_t totals_records(int wgs, int groups, bool wide) {
+  if (wide) return (size_t)groups;
+  return (size_t)std::max(groups, TOTALS_COPIES * std::min(groups, (wgs + 31) / 32));
+}
+
 size_t workspace_bytes_for(int P, int wgs, int groups, bool wide) {
   const size_t slot = exchange_slot_floats(P, wide);
   size_t bytes = STATUS_WORDS * sizeof(unsigned);
   bytes += (size_t)(wgs + 31) / 32 * 32 * sizeof(unsigned long long);
   bytes += (size_t)wgs * 2 * slot * sizeof(float);
-  bytes += (size_t)groups * slot * sizeof(float);
+  bytes += totals_records(wgs, groups, wide) * slot * sizeof(float);
   bytes += (size_t)groups * BARRIER_STRIDE_WORDS * sizeof(unsigned);
   return bytes;
 }
@@ -281,7 +288,7 @@ Workspace carve_workspace(void* base, int P, int wgs, int groups, bool wide) {
   w.partials = (float*)b;
   b += (size_t)wgs * 2 * slot * sizeof(float);
   w.totals = (float*)b;
-  b += (size_t)groups * slot * sizeof(float);
+  b += totals_records(wgs, groups, wide) * slot * sizeof(float);
   w.barrier = (unsigned*)b;
   return w;
 }
@@ -293,7 +300,7 @@ hipError_t clear_exchange(const Workspace& w, const KArgs& a, int groups, bool w
   if (wide) return launch_fill_u32(w.barrier, (size_t)groups * BARRIER_STRIDE_WORDS, 0u, st);
   hipError_t rc = launch_fill_u32((unsigned*)w.partials, (size_t)groups * 2 * a.G * w.slot_floats, 0u, st);
   if (rc == hipSuccess && a.two_phase)
-    rc = launch_fill_u32((unsigned*)w.totals, (size_t)groups * w.slot_floats, 0u, st);
+    rc = launch_fill_u32((unsigned*)w.totals, (size_t)groups * TOTALS_COPIES * w.slot_floats, 0u, st);
   return rc;
 }
 

@@ -46,6 +46,12 @@ enum KernelMode : int {
 // terms); rounded up to whole 128-byte lines so that a 32-parameter slice of a record is one line.
 inline int partial_slot_floats(int P) { return (((P + 3) / 4) * 4 + 4 + 31) / 32 * 32; }
 
+// 22 -> 40 -> 1 kernel, reduction by slices: the reducing workgroups publish the totals in up to this
+// many identical copies (one per 32 workgroups of the group) and workgroup `rank` polls copy
+// rank % copies, so that the polls of a group of 256 workgroups spread over eight times as many lines
+// (polls of one line are served one after the other).
+constexpr int TOTALS_COPIES = 8;
+
 // status words at the start of the exchange scratch (64 are reserved)
 constexpr int STATUS_WORDS = 64;
 

@@ -14,6 +14,8 @@
 // sample store of main_loop (include/mcmc/main.h:204-287).
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "bnn_device.h"
 #include "bnn_kernel_common.h"
 #include "bnn_kernels.h"
@@ -400,17 +402,23 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       ++bar_epoch;
       unsigned long long* my_part = part_base + ((size_t)buf * a.G + rank) * SLOT;
       if (rank != a.debug_drop_rank) {
+        // (all reads of the waves' slots are issued before the first addition: one LDS latency, not W)
+        float sv[PPT][W];
+#pragma unroll
+        for (int i = 0; i < PPT; ++i) {
+          const int p = min(tid + i * T, P - 1);
+#pragma unroll
+          for (int wv = 0; wv < W; ++wv) sv[i][wv] = s_slots[wv][p];
+        }
+        keep_together(sv);
 #pragma unroll
         for (int i = 0; i < PPT; ++i) {
           const int p = tid + i * T;
           if (p < P_AL) {
-            float v = 0.0f;
-            if (p < P) {
-              v = s_slots[0][p];
+            float v = sv[i][0];
 #pragma unroll
-              for (int wv = 1; wv < W; ++wv) v += s_slots[wv][p];
-            }
-            st_packet(my_part + p, v, epoch);
+            for (int wv = 1; wv < W; ++wv) v += sv[i][wv];
+            st_packet(my_part + p, p < P ? v : 0.0f, epoch);
           }
         }
         if (last && tid == 0) {
@@ -445,7 +453,6 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         for (int msk = 1; msk < 64; msk <<= 1) d += shfl_xor_d(d, msk);
         return d;
       };
-      constexpr int N_RED = (P_AL + 31) / 32;
       if (!a.two_phase) {
         // ---- stage 2 (small groups): every workgroup adds the G records.  A thread takes 16-byte
         //      columns (two parameters) of the records, eight loads in flight, records in ascending
@@ -476,65 +483,111 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
           if ((tid & 63) == 0) s_dl = d;
         }
       } else {
-        // ---- stage 2 (large groups), in two phases.  Phase 1: workgroup `rank` < ceil(P / 32) reduces
-        //      the 32-parameter slice [32 rank, 32 rank + 32) -- 256 bytes of every record -- over all
-        //      G records: thread (record lane rl = tid / 16, 16-byte column c = tid % 16) adds records
-        //      rl, rl + T/16, ... in order, the record lanes of a wave are added by a fixed xor tree and
-        //      the waves in order through LDS; the totals go out as flagged packets.  Phase 2: everyone
-        //      polls the totals. ----
-        unsigned long long* tot = reinterpret_cast<unsigned long long*>(a.totals) + (size_t)group * SLOT;
-        constexpr int RL = T / 16;  // record lanes of a workgroup
-        const bool reducer = rank < N_RED;
-        if (reducer) {
-          const int c = tid & 15, rl = tid >> 4;
-          const bool col_ok = 32 * rank + 2 * c < P_AL;  // P_AL is even: a column is whole or absent
-          const unsigned long long* src = grp_part + 32 * rank + 2 * c;
+        // ---- stage 2 (large groups), in two phases.  Phase 1: workgroup `rank` < ceil(P / SL) reduces
+        //      the SL-parameter slice [SL rank, SL rank + SL) over all G records: thread (record lane
+        //      rl = tid / CS, 16-byte column c = tid % CS, CS = SL / 2) adds records rl, rl + T / CS, ...
+        //      in order, the record lanes of a wave are added by a fixed xor tree and the waves in order
+        //      through LDS; the totals go out as flagged packets.  Phase 2: everyone polls the totals. ----
+        unsigned long long* tot_all =
+            reinterpret_cast<unsigned long long*>(a.totals) + (size_t)group * TOTALS_COPIES * SLOT;
+        // one copy per 32 workgroups of the group (a group of 32 polls its single copy as it stands)
+        const int copies = min(TOTALS_COPIES, a.G >> 5);
+        const unsigned long long* tot = tot_all + (size_t)(rank % copies) * SLOT;  // the copy this rank polls
+        // The wider the group, the narrower the slices and the more reducers: what bounds the first
+        // hand-off is the time one workgroup needs to pull its slice of every record through its own
+        // memory path (G x 256 bytes for a 32-parameter slice), and a poll that comes too early repeats
+        // all of it.  From 64 workgroups on the slices are 16 parameters wide (one 128-byte line of every
+        // record, 61 reducers), below that 32 (31 reducers).  Measured, ms per 1000 steps of one chain,
+        // slices of 32 / 16 / 8 parameters: G = 256: 9.31 / 9.25 / 9.47, G = 128: 11.84 / 11.56 / 12.12,
+        // G = 64: 17.01 / 16.75 / -.
+        const int CSr = a.G >= 64 ? 8 : 16;  // 16-byte columns per slice
+        const int SL = 2 * CSr;                                  // parameters per slice
+        const int n_red = (P_AL + SL - 1) / SL;
+        const bool reducer = rank < n_red;
+        auto reduce_slice = [&](auto cs_c, auto nb_c) {
+          constexpr int CS = decltype(cs_c)::value;
+          constexpr int RL = T / CS;                   // record lanes of a workgroup
+          constexpr int NB = decltype(nb_c)::value;    // records per thread and poll
+          const int c = tid & (CS - 1), rl = tid / CS;
+          const bool col_ok = 2 * CS * rank + 2 * c < P_AL;  // P_AL is even: a column is whole or absent
+          const unsigned long long* src = grp_part + 2 * CS * rank + 2 * c;
           float v0 = 0.0f, v1 = 0.0f;
-          for (int r0 = rl; r0 < a.G; r0 += 8 * RL) {
+          for (int r0 = rl; r0 < a.G; r0 += NB * RL) {
             f4 t8[8];
             const unsigned long long* p8[8];
             int valid = 0;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
-              p8[k] = src + (size_t)min(r0 + RL * k, a.G - 1) * SLOT;
-              if (r0 + RL * k < a.G) valid = k + 1;
+              p8[k] = src + (size_t)min(r0 + RL * (k < NB ? k : 0), a.G - 1) * SLOT;
+              if (k < NB && r0 + RL * k < a.G) valid = k + 1;
             }
-            wait_packets4x8(t8, p8, col_ok ? valid : 0, epoch, a.status, a.spin_limit, fine);
+            wait_packets4x8<NB>(t8, p8, col_ok ? valid : 0, epoch, a.status, a.spin_limit, fine);
 #pragma unroll
-            for (int k = 0; k < 8; ++k)
+            for (int k = 0; k < NB; ++k)
               if (k < valid) {
                 v0 += t8[k][0];
                 v1 += t8[k][2];
               }
           }
-          v0 += __shfl_xor(v0, 16);
-          v0 += __shfl_xor(v0, 32);
-          v1 += __shfl_xor(v1, 16);
-          v1 += __shfl_xor(v1, 32);
-          if ((tid & 63) < 16) {
+          // the record lanes of a wave (lanes that differ in the bits above the column index)
+#pragma unroll
+          for (int msk = CS; msk < 64; msk <<= 1) {
+            v0 += __shfl_xor(v0, msk);
+            v1 += __shfl_xor(v1, msk);
+          }
+          if ((tid & 63) < CS) {
             s_red2[wave][2 * c] = v0;
             s_red2[wave][2 * c + 1] = v1;
           }
+        };
+        if (reducer) {
+          // as many loads in flight per thread as it has records (at most eight a poll)
+          const int per_thread = (a.G * CSr + T - 1) / T;
+          using std::integral_constant;
+          if (CSr == 8) {
+            if (per_thread <= 2) reduce_slice(integral_constant<int, 8>{}, integral_constant<int, 2>{});
+            else if (per_thread <= 4) reduce_slice(integral_constant<int, 8>{}, integral_constant<int, 4>{});
+            else reduce_slice(integral_constant<int, 8>{}, integral_constant<int, 8>{});
+          } else {
+            if (per_thread <= 2) reduce_slice(integral_constant<int, 16>{}, integral_constant<int, 2>{});
+            else if (per_thread <= 4) reduce_slice(integral_constant<int, 16>{}, integral_constant<int, 4>{});
+            else reduce_slice(integral_constant<int, 16>{}, integral_constant<int, 8>{});
+          }
         }
         __syncthreads();
-        if (reducer && tid < 32 && 32 * rank + tid < P_AL && rank != a.debug_drop_rank) {
-          float x = s_red2[0][tid];
+        static_assert(T >= 32 * TOTALS_COPIES, "one thread per parameter of the slice and copy");
+        if (reducer && tid < SL * copies && SL * rank + (tid & (SL - 1)) < P_AL && rank != a.debug_drop_rank) {
+          const int pp = tid & (SL - 1), copy = tid / SL;
+          float rv[1][W];
 #pragma unroll
-          for (int wv = 1; wv < W; ++wv) x += s_red2[wv][tid];
-          st_packet(tot + 32 * rank + tid, x, epoch);
+          for (int wv = 0; wv < W; ++wv) rv[0][wv] = s_red2[wv][pp];
+          keep_together(rv);
+          float x = rv[0][0];
+#pragma unroll
+          for (int wv = 1; wv < W; ++wv) x += rv[0][wv];
+          st_packet(tot_all + (size_t)copy * SLOT + SL * rank + pp, x, epoch);
         }
-        if (last && rank == N_RED - 1 && wave == W - 1) {
+        if (last && rank == n_red - 1 && wave == W - 1) {
           const double d = sum_dl();
           if ((tid & 63) == 0) {
             const uint64_t bits = double_to_bits(d);
-            st_packet(tot + P_AL, __builtin_bit_cast(float, (uint32_t)bits), epoch);
-            st_packet(tot + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)), epoch);
+            for (int copy = 0; copy < copies; ++copy) {
+              unsigned long long* tc = tot_all + (size_t)copy * SLOT;
+              st_packet(tc + P_AL, __builtin_bit_cast(float, (uint32_t)bits), epoch);
+              st_packet(tc + P_AL + 1, __builtin_bit_cast(float, (uint32_t)(bits >> 32)), epoch);
+            }
           }
         }
-#pragma unroll
-        for (int i = 0; i < PPT; ++i) {
-          const int p = tid + i * T;
-          if (p < P) s_sum[p] = wait_packet(tot + p, epoch, a.status, a.spin_limit, fine);
+        // (the totals cannot be there before the reducers have seen every record: a workgroup that has
+        // nothing to reduce waits about a microsecond before its first poll instead of loading the
+        // memory system with polls that must fail)
+        if (!reducer) __builtin_amdgcn_s_sleep(48);
+        // a thread polls one 16-byte column (two packets) of the totals: one memory round trip
+        constexpr int NCOL = P_AL / 2;
+        for (int col = tid; col < NCOL; col += T) {
+          const f4 t4 = wait_packets4(tot + 2 * col, epoch, a.status, a.spin_limit, fine);
+          s_sum[2 * col] = t4[0];
+          s_sum[2 * col + 1] = t4[2];
         }
         if (last && tid == 0) {
           const float lo = wait_packet(tot + P_AL, epoch, a.status, a.spin_limit, fine);

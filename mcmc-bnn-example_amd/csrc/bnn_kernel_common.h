@@ -25,6 +25,31 @@ __device__ __forceinline__ int opaque_tid() {
   return t;
 }
 
+// A point all values of a row of `v` must have reached before anything computed from them starts (one
+// assembly statement that takes them all): placed between a batch of loads and the arithmetic on them,
+// it keeps the compiler from reading and adding one value at a time (a chain of load latencies).
+template <int A, int B>
+__device__ __forceinline__ void keep_together(float (&v)[A][B]) {
+  static_assert(B == 4 || B == 8 || B == 12 || B == 16, "rows of 4, 8, 12 or 16 values");
+#pragma unroll
+  for (int i = 0; i < A; ++i) {
+    float(&r)[B] = v[i];
+    if constexpr (B == 4) {
+      asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]));
+    } else if constexpr (B == 8) {
+      asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
+    } else if constexpr (B == 12) {
+      asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]),
+                        "+v"(r[8]), "+v"(r[9]), "+v"(r[10]), "+v"(r[11]));
+    } else {
+      // an assembly statement takes at most 30 operands (a read-write one counts twice)
+      asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]),
+                        "+v"(r[8]), "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]), "+v"(r[13]), "+v"(r[14]));
+      asm volatile("" : "+v"(r[15]));
+    }
+  }
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
   return __builtin_bit_cast(
@@ -38,6 +63,21 @@ __device__ __forceinline__ float row16_allreduce(float v) {
   v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
   v += dpp_move<0x141>(v);  // row_half_mirror
   v += dpp_move<0x140>(v);  // row_mirror
+  return v;
+}
+// the same for a double (its two halves moved separately)
+template <int CTRL>
+__device__ __forceinline__ double dpp_move_d(double v) {
+  const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+  const unsigned lo = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)b, CTRL, 0xf, 0xf, true);
+  const unsigned hi = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)(b >> 32), CTRL, 0xf, 0xf, true);
+  return __builtin_bit_cast(double, ((unsigned long long)hi << 32) | lo);
+}
+__device__ __forceinline__ double row16_allreduce_d(double v) {
+  v += dpp_move_d<0xB1>(v);
+  v += dpp_move_d<0x4E>(v);
+  v += dpp_move_d<0x141>(v);
+  v += dpp_move_d<0x140>(v);
   return v;
 }
 // Four sums over the 16 lanes of a DPP row at once, in 8 instructions instead of 4 x 4: the four
@@ -181,6 +221,35 @@ __device__ __forceinline__ void ld_agent4x8(f4 (&t)[8], const float* const (&p)[
       : "memory");
 }
 
+// the same with N = 1, 2 or 4 loads (the addresses p[N ..] are not touched)
+template <int N>
+__device__ __forceinline__ void ld_agent4xN(f4 (&t)[8], const float* const (&p)[8]) {
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8, "1, 2, 4 or 8 loads");
+  if constexpr (N == 8) {
+    ld_agent4x8(t, p);
+  } else if constexpr (N == 4) {
+    asm volatile(
+        "global_load_dwordx4 %0, %4, off sc1\n\t"
+        "global_load_dwordx4 %1, %5, off sc1\n\t"
+        "global_load_dwordx4 %2, %6, off sc1\n\t"
+        "global_load_dwordx4 %3, %7, off sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(t[0]), "=&v"(t[1]), "=&v"(t[2]), "=&v"(t[3])
+        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3])
+        : "memory");
+  } else if constexpr (N == 2) {
+    asm volatile(
+        "global_load_dwordx4 %0, %2, off sc1\n\t"
+        "global_load_dwordx4 %1, %3, off sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(t[0]), "=&v"(t[1])
+        : "v"(p[0]), "v"(p[1])
+        : "memory");
+  } else {
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(t[0]) : "v"(p[0]) : "memory");
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Per-wave working set handed to a layer for one leapfrog step
 // ------------------------------------------------------------------------------------------------
@@ -276,18 +345,20 @@ __device__ __forceinline__ float wait_packet(const unsigned long long* p, unsign
 __device__ __forceinline__ unsigned float_bits(float f) { return __builtin_bit_cast(unsigned, f); }
 // Eight 16-byte columns (two packets each) of up to eight records, polled until every packet of the
 // first `valid` records carries `flag`.
+// N = 1, 2, 4 or 8 loads per poll: only t[0 .. N) and p[0 .. N) are used.
+template <int N = 8>
 __device__ __forceinline__ void wait_packets4x8(f4 (&t)[8], const unsigned long long* const (&p)[8], int valid,
                                                 unsigned flag, unsigned* status, unsigned spin_limit,
                                                 bool& fine) {
   const float* q[8];
 #pragma unroll
-  for (int k = 0; k < 8; ++k) q[k] = reinterpret_cast<const float*>(p[k]);
+  for (int k = 0; k < 8; ++k) q[k] = reinterpret_cast<const float*>(p[k < N ? k : 0]);
   unsigned polls = 0;
   for (;;) {
-    ld_agent4x8(t, q);
+    ld_agent4xN<N>(t, q);
     bool ok = true;
 #pragma unroll
-    for (int k = 0; k < 8; ++k)
+    for (int k = 0; k < N; ++k)
       if (k < valid)
         ok = ok && float_bits(t[k][1]) == flag && float_bits(t[k][3]) == flag;
     if (ok) break;
@@ -296,6 +367,23 @@ __device__ __forceinline__ void wait_packets4x8(f4 (&t)[8], const unsigned long 
       break;
     }
   }
+}
+
+// One 16-byte column (two packets), polled until both packets carry `flag`.  Load and wait form one
+// assembly statement, as in ld_agent4x8.
+__device__ __forceinline__ f4 wait_packets4(const unsigned long long* p, unsigned flag, unsigned* status,
+                                            unsigned spin_limit, bool& fine) {
+  f4 t;
+  unsigned polls = 0;
+  for (;;) {
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(t) : "v"(p) : "memory");
+    if (float_bits(t[1]) == flag && float_bits(t[3]) == flag) break;
+    if (!poll_again(polls, status, spin_limit)) {
+      fine = false;
+      break;
+    }
+  }
+  return t;
 }
 
 // `epoch` counts the barriers of this launch from 1.  Up to 64 workgroups add to the group's counter

@@ -115,11 +115,10 @@ struct MfmaLayer {
       const int cc = cv ? c : 0;
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
+        // (one unconditional read per slot: a read under a lane mask would be waited for on its own)
         const int kk = KS * q + s;
-        float v = 0.0f;
-        if (kk < D0) v = s_w[kk * D1 + cc];
-        else if (kk == D0) v = s_w[oB1 + cc];
-        w1b[s][t] = cv ? v * kExp2Scale : 0.0f;
+        const float v = s_w[kk < D0 ? kk * D1 + cc : oB1 + cc];  // kk == D0: the bias row; beyond: padding
+        w1b[s][t] = cv && kk <= D0 ? v * kExp2Scale : 0.0f;
       }
       const float w2c = cv ? s_w[oW2 + cc] : 0.0f;
       w2lane += (double)w2c;
@@ -133,9 +132,7 @@ struct MfmaLayer {
     // added after the row sum, together with the target.
     const double share = (w2lane - (n == 0 ? (double)s_w[oB2] : 0.0)) * (double)k2;
     y_0 = (float)share;
-    double rest = share - (double)y_0;
-#pragma unroll
-    for (int msk = 1; msk < 16; msk <<= 1) rest += shfl_xor_d(rest, msk);
+    const double rest = row16_allreduce_d(share - (double)y_0);
     rho = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, (float)rest)));
     k2v = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, k2)));
   }
