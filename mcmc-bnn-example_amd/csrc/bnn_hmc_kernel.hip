@@ -168,6 +168,13 @@ struct FfmaLayer {
     return v;
   }
 
+  // a wave's slot in LDS is indexed by canonical parameter number, the log-likelihood difference behind
+  static constexpr int LDS_SLOT = (P_AL + 4 + 31) / 32 * 32;
+  static constexpr int DL_INDEX = P_AL;
+  static __device__ __forceinline__ int slot_index(int p) { return p; }
+  template <int LIK>
+  __device__ __forceinline__ float finish(int, float v, const float*) const { return v; }
+
   template <int LIK>
   __device__ __forceinline__ void write_partials(float* slot, const float*, bool) {
     const int lane = threadIdx.x & 63, cc = lane & 7, rg = lane >> 3;
@@ -224,7 +231,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   constexpr int PPT = (P + T - 1) / T;
 
   __shared__ float s_w[P_AL];
-  __shared__ __align__(16) float s_slots[W][SLOT];
+  __shared__ __align__(16) float s_slots[W][Layer::LDS_SLOT];
   __shared__ double s_red[W];
   __shared__ unsigned long long s_hash[W];
   __shared__ int s_progress[W];
@@ -406,9 +413,9 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
         float sv[PPT][W];
 #pragma unroll
         for (int i = 0; i < PPT; ++i) {
-          const int p = min(tid + i * T, P - 1);
+          const int idx = Layer::slot_index(min(tid + i * T, P - 1));
 #pragma unroll
-          for (int wv = 0; wv < W; ++wv) sv[i][wv] = s_slots[wv][p];
+          for (int wv = 0; wv < W; ++wv) sv[i][wv] = s_slots[wv][idx];
         }
         keep_together(sv);
 #pragma unroll
@@ -418,15 +425,15 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
             float v = sv[i][0];
 #pragma unroll
             for (int wv = 1; wv < W; ++wv) v += sv[i][wv];
-            st_packet(my_part + p, p < P ? v : 0.0f, epoch);
+            st_packet(my_part + p, p < P ? layer.template finish<LIK>(p, v, s_w) : 0.0f, epoch);
           }
         }
         if (last && tid == 0) {
           double d = 0.0;
 #pragma unroll
           for (int wv = 0; wv < W; ++wv) {
-            const uint64_t bits = ((uint64_t)__builtin_bit_cast(uint32_t, s_slots[wv][P_AL + 1]) << 32) |
-                                  __builtin_bit_cast(uint32_t, s_slots[wv][P_AL]);
+            const uint64_t bits = ((uint64_t)__builtin_bit_cast(uint32_t, s_slots[wv][Layer::DL_INDEX + 1]) << 32) |
+                                  __builtin_bit_cast(uint32_t, s_slots[wv][Layer::DL_INDEX]);
             d += bits_to_double(bits);
           }
           const uint64_t bits = double_to_bits(d);

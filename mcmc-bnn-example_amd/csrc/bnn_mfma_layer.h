@@ -710,80 +710,73 @@ struct MfmaLayer {
     return a + b;
   }
 
-  // this wave's partial sums -> its LDS slot, indexed by canonical parameter number; the factors
-  // 4 w2[c] left out of the GEMM2 operand and k / k2 left out of g are applied here.  `last`: the
-  // log-likelihood difference of the step is written too.
+  // ---- the wave's partial sums in LDS ----
+  // A wave's slot is a table of 48-float rows: row f < D0 holds the sums for feature f, row D0 those of
+  // the bias, row 24 those of the layer-2 weights, row 25 the log-likelihood difference; column c is
+  // the hidden unit (columns D1 .. 47 are the padded units: the first of them, in the bias row, holds the
+  // sum for b2).  With rows of 48 every lane stores whole registers unconditionally.
+  static constexpr int ROW = 16 * NT;
+  static constexpr int W2_ROW = 24, DL_ROW = 25;
+  static constexpr int LDS_SLOT = (DL_ROW + 1) * ROW;
+  static constexpr int DL_INDEX = DL_ROW * ROW;
+  static __device__ __forceinline__ int slot_index(int p) {
+    if (p < oW2) return (p / D1) * ROW + p % D1;  // W1 rows, then the bias row (oB1 = D0 D1)
+    if (p < oB2) return W2_ROW * ROW + (p - oW2);
+    return D0 * ROW + D1;
+  }
+  // What a sum over the waves' slots still lacks: the factors 4 w2[c] left out of the GEMM2 operand and
+  // k / k2 left out of g (applied once per workgroup, after the sum, not once per wave).
   template <int LIK>
-  __device__ __forceinline__ void write_partials(float* slot, const float* s_w, bool last) {
+  __device__ __forceinline__ float finish(int p, float v, const float* s_w) const {
+    const float gr = LIK == 1 ? ratio : 1.0f;
+    if (p < oW2) return v * (4.0f * gr * s_w[oW2 + p % D1]);
+    if (p < oB2) return v * gr;
+    return v * (4.0f * gr);
+  }
+
+  // this wave's partial sums -> its LDS slot (layout above).  `last`: the log-likelihood difference of
+  // the step is written too.
+  template <int LIK>
+  __device__ __forceinline__ void write_partials(float* slot, const float*, bool last) {
     const int lane = opaque_tid() & 63, n = lane & 15, q = lane >> 4;
     static_assert(D1 % 16 != 0, "db2 rides in the first padded hidden unit");
     static_assert(NT == 3, "the row-group sums below are laid out for three hidden tiles");
-    const float gr = LIK == 1 ? ratio : 1.0f;
-    const float gr4 = 4.0f * gr;
+    static_assert(D0 + 2 <= W2_ROW, "feature rows end below the layer-2 row");
     // The accumulators of features 16 .. D0 + 1 and of dw2 hold one partial per row group q (the four
     // rows of 16 lanes); two folds add the four partials of four registers at once and leave each row
     // of lanes with the total of one of them.  After
     //     fold16(fold32(x0, y0), fold32(x1, y1))
     // row q holds the total of (q & 1 ? x1 : x0) for q < 2 and of (q & 1 ? y1 : y0) for q >= 2,
     // added as (q0 + q2) + (q1 + q3).
-    // ---- factors first, so that the LDS reads are all in flight together ----
-    float fe[NT][4], ff[NT][4];
-    const int cb = 4 * (n >> 2) + (q & 1);  // features 16 ..: hidden unit of this lane after the folds
+    // ---- features 0 .. 15: lane (n, q), component i: c = 16 t + 4 q + i, f = n ----
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      *reinterpret_cast<f4*>(slot + n * ROW + 16 * t + 4 * q) = dacc_e[t];
+    // ---- features 16 .. D0 + 1: before the folds lane (n, q), component i holds
+    //      c = 16 t + 4 (n >> 2) + i, f = 16 + 2 (n & 3) + fb for row group q; after them the lane
+    //      holds c = 16 t + cb + 2 h and f = 16 + 2 (n & 3) + (q >> 1).  f = D0 is the bias; the sum of g
+    //      over the wave's rows (db2) has gathered in the first padded hidden unit ----
+    const int cb = 4 * (n >> 2) + (q & 1);
     const int f = 16 + 2 * (n & 3) + (q >> 1);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int ce = 16 * t + 4 * q + i, cf = 16 * t + 4 * (n >> 2) + i;
-        fe[t][i] = s_w[oW2 + min(ce, D1 - 1)];
-        ff[t][i] = s_w[oW2 + min(cf, D1 - 1)];
-      }
-    }
-    // ---- features 0 .. 15: lane (n, q), component i: c = 16 t + 4 q + i, f = n ----
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int c = 16 * t + 4 * q + i;
-        if (c < D1) slot[n * D1 + c] = dacc_e[t][i] * (gr4 * fe[t][i]);
-      }
-    }
-    // ---- features 16 .. D0 + 1: before the folds lane (n, q), component i holds
-    //      c = 16 t + 4 (n >> 2) + i, f = 16 + 2 (n & 3) + fb for row group q; after them the lane
-    //      holds c = 16 t + cb + 2 h and the f above.  f = D0 is the bias; the sum of g over the wave's
-    //      rows (db2) has gathered in the first padded hidden unit ----
-    const int fbase = f < D0 ? f * D1 : oB1;
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      float vs[2][4];  // scaled before the folds: the factor depends on (n, i) only
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int cf = 16 * t + 4 * (n >> 2) + i;
-        const float fac = gr4 * (cf < D1 ? ff[t][i] : 1.0f);
-        vs[0][i] = dacc_f[t][0][i] * fac;
-        vs[1][i] = dacc_f[t][1][i] * fac;
-      }
-#pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const float v = fold16(fold32(vs[0][2 * h], vs[1][2 * h]), fold32(vs[0][2 * h + 1], vs[1][2 * h + 1]));
-        const int c = 16 * t + cb + 2 * h;
-        if (f <= D0) {
-          if (c < D1) slot[fbase + c] = v;
-          else if (c == D1 && f == D0) slot[oB2] = v;
-        }
+        const float v = fold16(fold32(dacc_f[t][0][2 * h], dacc_f[t][1][2 * h]),
+                               fold32(dacc_f[t][0][2 * h + 1], dacc_f[t][1][2 * h + 1]));
+        slot[f * ROW + 16 * t + cb + 2 * h] = v;
       }
     }
     // ---- dw2 = sum_rows g h = 2 (sum_rows g s - sum_rows g / 2); the second sum is what the first
     //      padded hidden unit (lane n = D1 % 16 of the last hidden tile, s = 1/2) has accumulated ----
     {
       const float half_gsum = dpp_move<0x150 + D1 % 16>(dw2s[NT - 1]);  // row_newbcast
-      const float v0 = 2.0f * (dw2s[0] - half_gsum) * gr;
-      const float v1 = 2.0f * (dw2s[1] - half_gsum) * gr;
-      const float v2 = 2.0f * (dw2s[2] - half_gsum) * gr;
+      const float v0 = 2.0f * (dw2s[0] - half_gsum);
+      const float v1 = 2.0f * (dw2s[1] - half_gsum);
+      const float v2 = 2.0f * (dw2s[2] - half_gsum);
       const float v = fold16(fold32(v0, v1), fold32(v2, v2));  // rows: tile 0, tile 2, tile 1, tile 2
       const int t = q == 0 ? 0 : (q == 2 ? 1 : 2);
-      const int c = 16 * t + n;
-      if (q < 3 && c < D1) slot[oW2 + c] = v;
+      slot[W2_ROW * ROW + 16 * t + n] = v;  // (rows 1 and 3 store the same bits to the same place)
     }
     if (last) {
       double d = dl;  // held by lanes n == 0
@@ -791,8 +784,8 @@ struct MfmaLayer {
       d += shfl_xor_d(d, 32);
       if (lane == 0) {
         const uint64_t bits = double_to_bits(d);
-        slot[P_AL] = __builtin_bit_cast(float, (uint32_t)bits);
-        slot[P_AL + 1] = __builtin_bit_cast(float, (uint32_t)(bits >> 32));
+        slot[DL_INDEX] = __builtin_bit_cast(float, (uint32_t)bits);
+        slot[DL_INDEX + 1] = __builtin_bit_cast(float, (uint32_t)(bits >> 32));
       }
     }
   }
