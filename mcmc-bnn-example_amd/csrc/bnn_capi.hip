@@ -304,6 +304,26 @@ hipError_t clear_exchange(const Workspace& w, const KArgs& a, int groups, bool w
   return rc;
 }
 
+// Host-side check before every launch: what the kernel of a launch of `groups` chain groups (a.G
+// workgroups each, `wgs` in all) will touch in the exchange scratch lies inside the scratch as it was
+// carved.  A launch that would not fit is refused, never started.
+int check_exchange_bounds(const Workspace& w, const void* base, size_t bytes, const KArgs& a, int groups, int wgs,
+                          bool wide) {
+  const char* end = (const char*)base + bytes;
+  const char* hash_end = (const char*)(w.rank_hash + wgs);
+  const char* part_end = (const char*)(w.partials + (size_t)groups * 2 * a.G * w.slot_floats);
+  const size_t tot_records = !a.two_phase ? 0 : (size_t)groups * (wide ? 1 : TOTALS_COPIES);
+  const char* tot_end = (const char*)(w.totals + tot_records * w.slot_floats);
+  const char* bar_end = (const char*)(w.barrier + (wide ? (size_t)groups * BARRIER_STRIDE_WORDS : 0));
+  if (hash_end > (const char*)w.partials || part_end > (const char*)w.totals || tot_end > (const char*)w.barrier ||
+      bar_end > end || (const char*)w.barrier > end)
+    return fail(BNNHMC_ERR_INVALID,
+                "internal: a launch of %d chain groups x %d workgroups does not fit the exchange scratch of "
+                "%zu bytes; not launched",
+                groups, a.G, bytes);
+  return BNNHMC_OK;
+}
+
 // Synchronises `stream` and reads the status words the launches on it have left since the words
 // were last cleared: BNNHMC_ERR_TIMEOUT if a bounded wait expired, BNNHMC_ERR_DIVERGED if the
 // workgroups of a chain group did not all hold the same state at the end of a launch.
@@ -574,8 +594,10 @@ int launch_and_count(bnnhmc_sampler* s, KArgs& a, int groups) {
   int wgs = 0;
   set_grid(a, groups, s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs, 256) : s->plan.G,
            s->plan.wide, &wgs);
-  HIP_TRY(clear_exchange(carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups, s->plan.wide),
-                         a, groups, s->plan.wide, s->stream));
+  const Workspace w = carve_workspace(s->workspace, s->L.P, s->plan.resident_wgs, s->plan.max_groups, s->plan.wide);
+  const int fits = check_exchange_bounds(w, s->workspace, s->workspace_bytes, a, groups, wgs, s->plan.wide);
+  if (fits != BNNHMC_OK) return fits;
+  HIP_TRY(clear_exchange(w, a, groups, s->plan.wide, s->stream));
   HIP_TRY(launch_hmc_kernel(s->plan.kernel, a, wgs, s->plan.threads, s->plan.dyn_lds, s->stream));
   HIP_TRY(launch_compare_hashes(a.rank_hash, wgs, a.G, a.status, s->stream));
   s->last_workgroups = wgs;
@@ -818,6 +840,8 @@ static int mcmc_step_on(const bnnhmc_model* model, const bnnhmc_launch* launch, 
   a.rank_hash = w.rank_hash;
   int wgs = 0;
   set_grid(a, 1, G, plan.wide, &wgs);
+  const int fits = check_exchange_bounds(w, workspace, workspace_bytes, a, 1, wgs, plan.wide);
+  if (fits != BNNHMC_OK) return fits;
   // status words and the exchange area start from zero on every call
   HIP_TRY(launch_fill_u32(w.status, STATUS_WORDS, 0u, st));
   HIP_TRY(clear_exchange(w, a, 1, plan.wide, st));
