@@ -198,3 +198,24 @@ def test_split_rhat_and_ess(lib, pkg):
     assert r1[0] < 1.02 and 0.6 * S < e1[0] < 1.4 * S
     with pytest.raises(pkg.BnnHmcError):
         lib.split_rhat_ess(xs[:, :7])
+
+
+def test_step_workspace_holds_what_the_exchange_needs(lib):
+    """Sizes from bnnhmc_step_workspace_bytes against what the exchange of the 22 -> 40 -> 1 kernel must
+    hold whatever its layout: two records (double buffer) of P eight-byte packets per workgroup, and
+    from 32 workgroups on at least one more such record for the totals; never less for more workgroups;
+    and every single-chain configuration up to 256 workgroups fits the 4.5 MiB static scratch of
+    bnnhmc_mcmc_step_static."""
+    m = lib.default_model()
+    P = lib.c.bnnhmc_num_params(m.d0, m.d1)
+    prev = 0
+    for G in (1, 2, 4, 8, 16, 32, 64, 128, 256):
+        launch = lib.default_launch(cus_per_chain=G)
+        n = lib.c.bnnhmc_step_workspace_bytes(C.byref(m), C.byref(launch))
+        need = 2 * G * P * 8 + (P * 8 if G >= 32 else 0) + 64 * 4
+        assert n >= need, (G, n, need)
+        assert n % 16 == 0 and n >= prev
+        assert n <= 4608 * 1024
+        prev = n
+    # the default of the step operator is the widest group
+    assert lib.c.bnnhmc_step_workspace_bytes(C.byref(m), C.byref(lib.default_launch())) == prev
