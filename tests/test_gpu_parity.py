@@ -63,7 +63,7 @@ def test_device_momentum_stream_is_bit_exact(lib, orc):
 @pytest.mark.parametrize("layer", ["mfma", "ffma"])
 @pytest.mark.parametrize("kind", ["t", "gauss"])
 @pytest.mark.parametrize("n,G", [(1, 1), (3, 2), (16, 1), (17, 4), (100, 3), (1000, 8), (4101, 32),
-                                 (58368, 32), (58368, 0), (9000, 96), (58368, 256)])
+                                 (58368, 32), (58368, 0), (9000, 96), (58368, 256), (6000, 48), (30000, 200)])
 def test_eval_matches_oracle(pkg, lib, orc, layer, kind, n, G):
     say("eval layer=%s lik=%s n=%d G=%d" % (layer, kind, n, G))
     model, om, gen = models(pkg, lib, kind, n)
