@@ -368,8 +368,9 @@ int widen_group(int G, int groups, int resident_wgs, int cap) {
 void set_grid(KArgs& a, int groups, int G, bool wide, int* workgroups) {
   const int wgs = groups * G;
   a.G = G;
-  // From 32 workgroups per chain on, each of the first 31 workgroups reduces one 32-parameter slice of
-  // the records and everyone reads the totals, instead of everyone reading every record.  Measured on
+  // From 32 workgroups per chain on, the first workgroups of a group each reduce one slice of the
+  // records (32 parameters, 31 reducers; from 64 workgroups on 16 parameters, 61 reducers) and everyone
+  // reads the totals, instead of everyone reading every record.  Measured on
   // MI355X with the 22 -> 40 -> 1 kernel (evaluations/s, all-read vs slices): G = 32: 278 k vs 288 k,
   // G = 64: 183 k vs 230 k.  The 64 -> 128 -> 1 kernel, whose hand-offs go through barriers, switches
   // above 64.
