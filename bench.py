@@ -112,6 +112,10 @@ def main():
     ap.add_argument("--full", action="store_true",
                     help="run the whole 200 windows x (100 + 800) transitions job from the all-zero start with "
                          "the reference's adaptation and time all of it")
+    ap.add_argument("--lik", choices=["gaussian", "student_t"], default="gaussian",
+                    help="gaussian = the benchmark configurations (sigma 0.01, prior N(0, 0.1^2)); student_t = the "
+                         "reference's own model constants (Student-t scale 100, 2.2 degrees of freedom, prior scale "
+                         "200) on the same synthetic data")
     ap.add_argument("--samples", type=int, default=800, choices=[800, 1600],
                     help="--full only: kept samples per window (800 = configs[2], 1600 = configs[3])")
     args = ap.parse_args()
@@ -152,8 +156,14 @@ def main():
     plan = batch_plan(n_chains, resident_wgs, launch.cus_per_chain, wide)
     resident = plan[0][0]                                   # chains in flight in the first launches
 
-    model = lib.default_model(d0=d0, d1=d1, n=n_rows, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01,
-                              prior_scale=0.1)
+    student = args.lik == "student_t"
+    if student:
+        model = lib.default_model(d0=d0, d1=d1, n=n_rows)  # global_params.h:39-48
+        if args.eps0 == 2e-5:
+            args.eps0 = 0.027  # what the adaptation reaches with this model on this data
+    else:
+        model = lib.default_model(d0=d0, d1=d1, n=n_rows, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01,
+                                  prior_scale=0.1)
     if args.full:
         burn, keep, adapt = 100, args.samples, 100
     else:  # warm-up = burn-in (nothing stored), timed transitions store their samples; no adaptation
@@ -233,11 +243,12 @@ def main():
         "config": {
             "workload": "configs[%s]: %d independent windows x %d chain(s), all resident in HBM (%d chains in "
                         "flight per launch), %d->%d->1 BNN, %dx%d features ~N(0,1), teacher-MLP targets + "
-                        "N(0,0.01^2), Gaussian likelihood and prior, %d leapfrog steps per transition; one step "
+                        "N(0,0.01^2), %s, %d leapfrog steps per transition; one step "
                         "= one transition of every window, samples stored in the timed region" % (
                             "4" if wide else ("3" if args.full and keep == 1600 else "2"), n_windows, cpw,
                             min(n_chains, resident), d0, d1, n_rows, d0,
-                            args.leapfrog),
+                            "Student-t likelihood (scale 100, 2.2 degrees of freedom) and prior scale 200 as in the "
+                            "reference" if student else "Gaussian likelihood and prior", args.leapfrog),
             "layer": args.layer, "wgs_per_cu": wgs_per_cu,
             "launches_chains_x_workgroups_per_chain": (
                 "%d x %d, the %d chains taking turns in quanta of %d transitions; what does not fill a launch runs "
