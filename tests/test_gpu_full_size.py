@@ -392,3 +392,36 @@ def test_single_chain_on_256_workgroups_soak(pkg, lib, orc):
     assert st["n_accepted"] > 20, st["n_accepted"]           # the adaptation got the chain going
     assert s.timing()["workgroups"] == 256
     s.close()
+
+
+def test_reference_model_first_transitions_at_full_size(pkg, lib, orc):
+    """The reference's own model constants (Student-t likelihood, scale 100, 2.2 degrees of freedom, prior scale
+    200: global_params.h:39-48) at full size, from the all-zero start with eps0 = 0.01 as main_loop does
+    (main.h:182-202): the first 12 transitions of 1000 leapfrog steps.  Decisions and the step-size trace must
+    equal the oracle's; this posterior is smooth at that step size (no transition diverges), so the log accept
+    ratios must agree as well, to the rounding noise of their row sums."""
+    say("reference model, 12 transitions of 1000 leapfrog steps at full size")
+    model = lib.default_model(n=N_FULL)
+    om = ob.ref_model(N_FULL)
+    hmc = lib.default_hmc(leapfrog_steps=L_FULL, burn_in=100, n_samples=4, eps0=0.01, seed=0)
+    oh = ob.ref_hmc(L_FULL, 100, 4, 0, 0, 0.01)
+    s = lib.create(model, hmc, lib.default_launch(), 1, 1)
+    s.generate_window(0, teacher_scale=0.1, noise_sigma=0.01)
+    X, y = s.get_window_data(0)
+    s.init_chains(None)
+    s.run(12)
+    tr = s.get_traces(0)
+    s.close()
+    t0 = time.time()
+    ref = orc.run_chain_from(om, oh, X, y, None, 0.01, 0, 12)
+    say("oracle: 12 transitions in %.1f s" % (time.time() - t0))
+    assert np.array_equal(tr["accept"][:12], ref["accept"])
+    assert tr["eps"][:12].tobytes() == ref["eps"].tobytes()
+    assert np.all(np.isfinite(ref["log_acpt"]))
+    err = np.abs(tr["log_acpt"][:12].astype(np.float64) - ref["log_acpt"])
+    say("log accept ratios: oracle %s, largest difference %.3g" % (np.array2string(ref["log_acpt"], precision=4),
+                                                                  err.max()))
+    # the ratios themselves are of order 1e-3 here.  Each is a sum of 58368 differences of per-row
+    # log-likelihoods of size 5.6, known to one FP32 ulp (4.8e-7): at random signs that is 1.2e-4 of rounding
+    # noise in either implementation (measured difference: 2.8e-5)
+    assert err.max() <= 2e-4
