@@ -77,7 +77,10 @@ typedef struct bnnhmc_launch {
                       /* more chains on 256 CUs: 2 each); more chains than fit take turns on such  */
                       /* batches, transitions_per_launch transitions at a time, and what does not  */
                       /* fill a batch runs in smaller, wider ones.  64 -> 128 -> 1: 4, a smaller    */
-                      /* last batch widened.  Step operator: 256                                    */
+                      /* last batch widened.  Step operator: 256.  Results are bit-reproducible for */
+                      /* a fixed count; with 0 and more chains than fit at once, which launches run */
+                      /* wider depends on how a job is cut into bnnhmc_run calls, so a run that     */
+                      /* must be repeatable or resumable bit for bit sets an explicit count         */
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */
   int threads;        /* threads per workgroup; default 512 for MFMA (every tile loop), 256 for  */
                       /* FFMA and with wgs_per_cu = 2.  The plain MFMA loop is also built for    */
@@ -88,7 +91,8 @@ typedef struct bnnhmc_launch {
                       /* asking for it with another size is an error),                           */
                       /* 1 = software-pipelined GEMM/pointwise stages (512 or 256 threads),      */
                       /* 3 = plain loop (256, 512, 768 or 1024 threads)                          */
-  int transitions_per_launch; /* bound on one kernel's run time (default 8; 1 for 64 -> 128 -> 1) */
+  int transitions_per_launch; /* bound on one kernel's run time (default 5; 1 for 64 -> 128 -> 1);       */
+                              /* times leapfrog_steps it must stay below 2^32 - 1                        */
   unsigned spin_limit; /* polls before an in-kernel wait gives up (default 1 << 22)              */
 } bnnhmc_launch;
 
@@ -111,6 +115,14 @@ int bnnhmc_device_info(int* n_devices, int* compute_units, char* arch, size_t ar
  * result is). */
 size_t bnnhmc_step_workspace_bytes(const bnnhmc_model* model, const bnnhmc_launch* launch);
 
+/* How the step operator lays one chain over the GPU: workgroups, threads per workgroup, the most rows a
+ * wavefront takes, LDS bytes of a workgroup and the most a workgroup may use.  Stands in for the
+ * compile-time constants N_BLKS, N_THREADS, N_WARP_SAMPLES and for full_smem_size<T>() /
+ * leapfrog_max_smem_size<T>() that the reference's driver prints (include/mcmc/main.h:120-125;
+ * include/mcmc/mcmc_step_ffma.h:46-70).  Any output may be NULL.  Needs a device. */
+int bnnhmc_step_launch_info(const bnnhmc_model* model, const bnnhmc_launch* launch, int* workgroups,
+                            int* threads, int* rows_per_wave, size_t* lds_bytes, size_t* lds_max_bytes);
+
 /* L fused leapfrog steps.  Replaces mcmc::mcmc_step<T, LP_STEPS>
  * (include/mcmc/mcmc_step_ffma.h:395-427, include/mcmc/mcmc_step_tc.h:679-696).
  * In : weights_prev, mom_prev, grad_prev (full gradient of the log-posterior at weights_prev), eps.
@@ -131,17 +143,22 @@ int bnnhmc_mcmc_step(const bnnhmc_model* model, const bnnhmc_launch* launch, con
  * has no counterpart in the reference.  Configurations whose scratch would not fit (see
  * bnnhmc_step_workspace_bytes) are refused with BNNHMC_ERR_INVALID.  All calls on one GPU share the
  * array: calls that overlap on one GPU (two streams, two threads) race; calls issued one after the
- * other on one stream do not.  Check the outcome with bnnhmc_step_check(model, launch, NULL, stream). */
+ * other on one stream do not.  Check the outcome with bnnhmc_step_check(model, launch, NULL, stream).
+ * The first call for a (device, model, launch) configuration looks up device properties, the kernel's
+ * occupancy and the array's address, none of which may be asked for while a stream is capturing: make
+ * one call per configuration outside capture first; every later call only launches kernels. */
 int bnnhmc_mcmc_step_static(const bnnhmc_model* model, const bnnhmc_launch* launch, const float* x,
                             const float* y, const float* weights_prev, float* weights_next,
                             const float* mom_prev, float* mom_next, const float* grad_prev,
                             float* grad_cur, float* grad_next, float* loss_values, float eps,
                             int lp_steps, void* stream);
 
-/* Synchronises `stream` and reports whether the last bnnhmc_mcmc_step on this workspace ran to
- * completion: BNNHMC_ERR_TIMEOUT if a bounded in-kernel wait expired (the outputs were then not
- * written), BNNHMC_ERR_DIVERGED if the workgroups did not all hold the same state at the end.  Every
- * bnnhmc_mcmc_step clears the record of the one before it, so check each step whose outcome matters.
+/* Synchronises `stream` and reports whether every bnnhmc_mcmc_step on this workspace since the last
+ * check ran to completion: BNNHMC_ERR_TIMEOUT if a bounded in-kernel wait expired (the outputs of that
+ * step were then not written, and steps queued behind it may have been abandoned too),
+ * BNNHMC_ERR_DIVERGED if the workgroups did not all hold the same state at the end of a step.  The
+ * record of a failure stays in the workspace until this call has reported it (and then clears it), so
+ * one check after a whole sequence of steps is enough.
  * `launch` is not needed (the record sits at the start of the workspace) and may be NULL; workspace
  * NULL means the library's own scratch (bnnhmc_mcmc_step_static) on the current GPU.  Stands in
  * for the CUDA_CHECK after the launch (include/mcmc/mcmc_step_ffma.h:412). */

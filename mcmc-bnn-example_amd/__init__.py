@@ -55,7 +55,7 @@ EXPORTS = [
     "bnnhmc_get_window_data", "bnnhmc_init_chains", "bnnhmc_run", "bnnhmc_get_samples",
     "bnnhmc_get_chain_state", "bnnhmc_get_traces", "bnnhmc_eval", "bnnhmc_final_loss",
     "bnnhmc_get_timing", "bnnhmc_read_reference_data", "bnnhmc_set_chain_state",
-    "bnnhmc_split_rhat_ess", "bnnhmc_window_diagnostics",
+    "bnnhmc_split_rhat_ess", "bnnhmc_window_diagnostics", "bnnhmc_step_launch_info",
 ]
 
 

@@ -33,6 +33,30 @@ hipError_t launch_fill_f32(float* p, size_t n, float v, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Status words of a step-operator workspace: cleared only when the workspace has not been used before
+// (it then holds whatever the caller's allocation held), which the last two status words tell: the
+// library leaves a 64-bit mark there once it has cleared the others.  A record of a failed step thus
+// stays until bnnhmc_step_check has reported it, however many steps were queued behind it.
+constexpr unsigned STATUS_MARK0 = 0x626e6e68u, STATUS_MARK1 = 0x6d637374u;
+__global__ void prepare_status_kernel(unsigned* status) {
+  const unsigned m0 = status[STATUS_WORDS - 2], m1 = status[STATUS_WORDS - 1];
+  __syncthreads();
+  if (m0 == STATUS_MARK0 && m1 == STATUS_MARK1) return;
+  const int t = (int)threadIdx.x;
+  if (t < STATUS_WORDS - 2) status[t] = 0u;
+  else if (t == STATUS_WORDS - 2) status[t] = STATUS_MARK0;
+  else if (t == STATUS_WORDS - 1) status[t] = STATUS_MARK1;
+}
+hipError_t launch_prepare_status(unsigned* status, hipStream_t stream) {
+  static_assert(STATUS_WORDS == 64, "one thread per status word");
+  hipLaunchKernelGGL(prepare_status_kernel, dim3(1), dim3(STATUS_WORDS), 0, stream, status);
+  return hipGetLastError();
+}
+// clears a reported record, leaving the mark in place
+hipError_t launch_clear_status(unsigned* status, hipStream_t stream) {
+  return launch_fill_u32(status, STATUS_WORDS - 2, 0u, stream);
+}
+
 // Runs after every launch of a trajectory kernel: all workgroups of a chain group must report the
 // same state hash.  The first mismatch is recorded in the status words ([4] workgroup index + 1,
 // [5] its chain group, [6..9] the two hashes); a launch that was abandoned (status[0] set) left no

@@ -136,7 +136,7 @@ struct Plan {
   int resident_wgs = 0;  // workgroups that can be co-resident on the device
   bool widen = false;    // default group size: a batch that leaves CUs idle gets wider groups
   unsigned spin_limit = 1u << 22;
-  int transitions_per_launch = 8;
+  int transitions_per_launch = 5;
 };
 
 int make_plan_uncached(const bnnhmc_model& m, const bnnhmc_launch* lp, const DeviceInfo& di, Plan& p) {
@@ -388,13 +388,15 @@ int debug_drop_rank() {
   return e && *e ? atoi(e) : -1;
 }
 
-// Test hook: BNNHMC_DEBUG_PERTURB_HASH=<rank> makes that rank of every chain group flip one bit of
-// the state hash it reports (its memory traffic and its results are untouched), so that the
-// comparison of the hashes fails.  Unset in normal use.
+// Measurement switch: BNNHMC_BALANCE=0 turns off the pacing of the two waves that share a SIMD (wave
+// priorities in the prefetched tile loop).  Unset in normal use (pacing on).
 int env_balance() {
   const char* e = getenv("BNNHMC_BALANCE");
   return e && *e ? atoi(e) : 1;
 }
+// Test hook: BNNHMC_DEBUG_PERTURB_HASH=<rank> makes that rank of every chain group flip one bit of
+// the state hash it reports (its memory traffic and its results are untouched), so that the
+// comparison of the hashes fails.  Unset in normal use.
 int debug_perturb_hash_rank() {
   const char* e = getenv("BNNHMC_DEBUG_PERTURB_HASH");
   return e && *e ? atoi(e) : -1;
@@ -674,7 +676,7 @@ void bnnhmc_default_launch(bnnhmc_launch* l) {
   l->wgs_per_cu = 1;
   l->threads = 0;
   l->pipeline = 0;
-  l->transitions_per_launch = 8;
+  l->transitions_per_launch = 5;
   l->spin_limit = 1u << 22;
 }
 
@@ -775,6 +777,34 @@ size_t bnnhmc_step_workspace_bytes(const bnnhmc_model* model, const bnnhmc_launc
   return workspace_bytes_for(make_layout(model->d0, model->d1).P, G, 1, model->d0 == 64 && model->d1 == 128);
 }
 
+int bnnhmc_step_launch_info(const bnnhmc_model* model, const bnnhmc_launch* launch, int* workgroups,
+                            int* threads, int* rows_per_wave, size_t* lds_bytes, size_t* lds_max_bytes) {
+  int rc = check_model(model);
+  if (rc) return rc;
+  DeviceInfo di;
+  rc = query_device(di);
+  if (rc) return rc;
+  Plan plan;
+  rc = make_plan(*model, launch, di, plan);
+  if (rc) return rc;
+  const int G = step_group(launch, plan.resident_wgs, 256);
+  const int waves = G * (plan.threads / 64), tiles = (model->n + 15) / 16;
+  if (workgroups) *workgroups = G;
+  if (threads) *threads = plan.threads;
+  if (rows_per_wave) *rows_per_wave = 16 * ((tiles + waves - 1) / waves);
+  if (lds_bytes || lds_max_bytes) {
+    hipFuncAttributes attr;
+    HIP_TRY(hipFuncGetAttributes(&attr, plan.kernel));
+    if (lds_bytes) *lds_bytes = attr.sharedSizeBytes + plan.dyn_lds;
+    if (lds_max_bytes) {
+      int v = 0;
+      HIP_TRY(hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, 0));
+      *lds_max_bytes = (size_t)v;
+    }
+  }
+  return BNNHMC_OK;
+}
+
 // The step operator on a given exchange scratch; allocates nothing (device and plan queries happen on
 // the first call for a configuration only, and allocate nothing either).
 static int mcmc_step_on(const bnnhmc_model* model, const bnnhmc_launch* launch, const float* x,
@@ -843,8 +873,9 @@ static int mcmc_step_on(const bnnhmc_model* model, const bnnhmc_launch* launch, 
   set_grid(a, 1, G, plan.wide, &wgs);
   const int fits = check_exchange_bounds(w, workspace, workspace_bytes, a, 1, wgs, plan.wide);
   if (fits != BNNHMC_OK) return fits;
-  // status words and the exchange area start from zero on every call
-  HIP_TRY(launch_fill_u32(w.status, STATUS_WORDS, 0u, st));
+  // The exchange area starts from zero on every call.  The status words are cleared on the first use
+  // of a workspace only: the record of a step that failed stays until bnnhmc_step_check reports it.
+  HIP_TRY(launch_prepare_status(w.status, st));
   HIP_TRY(clear_exchange(w, a, 1, plan.wide, st));
   HIP_TRY(launch_hmc_kernel(plan.kernel, a, wgs, plan.threads, plan.dyn_lds, st));
   HIP_TRY(launch_compare_hashes(a.rank_hash, wgs, G, a.status, st));
@@ -888,7 +919,15 @@ int bnnhmc_step_check(const bnnhmc_model* model, const bnnhmc_launch* launch, vo
     if (rc) return rc;
   }
   // the status words sit at the start of the workspace whatever the launch parameters were
-  return read_status(workspace, (hipStream_t)stream);
+  const int rc = read_status(workspace, (hipStream_t)stream);
+  if (rc == BNNHMC_ERR_TIMEOUT || rc == BNNHMC_ERR_DIVERGED) {
+    // reported once: the record is cleared so that the workspace can be used again
+    const std::string msg = g_last_error;
+    HIP_TRY(launch_clear_status((unsigned*)workspace, (hipStream_t)stream));
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    g_last_error = msg;
+  }
+  return rc;
 }
 
 int bnnhmc_sample_momentum(uint32_t seed, uint32_t chain_id, uint32_t transition, int n,
@@ -951,6 +990,17 @@ int bnnhmc_create(const bnnhmc_model* model, const bnnhmc_hmc* hmc, const bnnhmc
     return fail(BNNHMC_ERR_INVALID, "bad sampler constants");
   if (n_windows < 1 || chains_per_window < 1)
     return fail(BNNHMC_ERR_INVALID, "n_windows and chains_per_window must be >= 1");
+  {
+    // the exchange numbers the leapfrog steps of a launch in 32 bits, from 1 (0 = the cleared state)
+    bnnhmc_launch dl;
+    bnnhmc_default_launch(&dl);
+    const long long tpl = launch && launch->transitions_per_launch > 0 ? launch->transitions_per_launch
+                                                                         : dl.transitions_per_launch;
+    if (tpl * (long long)hmc->leapfrog_steps >= 0xFFFFFFFFll)
+      return fail(BNNHMC_ERR_INVALID,
+                  "transitions_per_launch (%lld) x leapfrog_steps (%d) must stay below 2^32 - 1", tpl,
+                  hmc->leapfrog_steps);
+  }
   DeviceInfo di;
   rc = query_device(di);
   if (rc) return rc;

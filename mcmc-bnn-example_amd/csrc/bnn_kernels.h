@@ -21,6 +21,10 @@ hipError_t launch_hmc_kernel(const void* kernel, const KArgs& args, int workgrou
 // small kernels
 hipError_t launch_fill_u32(unsigned* p, size_t n, unsigned v, hipStream_t stream);
 hipError_t launch_fill_f32(float* p, size_t n, float v, hipStream_t stream);
+// status words of a step-operator workspace: cleared on first use only (see prepare_status_kernel);
+// launch_clear_status clears a record that has been reported
+hipError_t launch_prepare_status(unsigned* status, hipStream_t stream);
+hipError_t launch_clear_status(unsigned* status, hipStream_t stream);
 // compares the state hashes the workgroups of the last trajectory launch reported (see
 // compare_hashes_kernel); status words as described there
 hipError_t launch_compare_hashes(const unsigned long long* h, int wgs, int G, unsigned* status,

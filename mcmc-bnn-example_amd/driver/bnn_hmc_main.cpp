@@ -162,9 +162,10 @@ int main(int argc, char** argv) {
   CHECK(bnnhmc_init_chains(s, nullptr));
 
   // ------------------------------------------------------------------ run (main.h:204-287)
-  // calls of whole launch quanta, long enough that chains which take turns on the device (more windows
-  // than fit at once) do so on full launches
-  const int total = hmc.burn_in + hmc.n_samples, every = 5 * launch.transitions_per_launch;
+  // calls of 100 transitions (a progress dot each): inside one call, chains that take turns on the device
+  // (more windows than fit at once) do so on launches that fill it, and only what is left at the end of a
+  // call runs in narrower ones, so long calls cost less than short ones
+  const int total = hmc.burn_in + hmc.n_samples, every = 100;
   for (int done = 0; done < total; done += every) {
     CHECK(bnnhmc_run(s, std::min(every, total - done)));
     std::printf(".");

@@ -16,6 +16,7 @@ def hip():
         _hip.hipFree.argtypes = [C.c_void_p]
         _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
         _hip.hipMemset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
+        _hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
     return _hip
 
 
@@ -61,6 +62,13 @@ class DevBuf:
             self.free()
         except Exception:
             pass
+
+
+def free_bytes():
+    """free device memory as the runtime reports it"""
+    free, total = C.c_size_t(), C.c_size_t()
+    _ok(hip().hipMemGetInfo(C.byref(free), C.byref(total)), "hipMemGetInfo")
+    return free.value
 
 
 def synchronize():

@@ -219,3 +219,40 @@ def test_step_workspace_holds_what_the_exchange_needs(lib):
         prev = n
     # the default of the step operator is the widest group
     assert lib.c.bnnhmc_step_workspace_bytes(C.byref(m), C.byref(lib.default_launch())) == prev
+
+
+def test_operator_header_compiles_with_the_host_compiler(pkg, tmp_path):
+    """include/mcmc_step_hip.h offers what the reference's driver takes from its operator header
+    (main.h:38-42, 52-59, 120-133; mcmc_step_ffma.h:46-70, 395-436).  Compiled here by g++ against
+    stand-ins for the reference's constants and its DeviceMatrix (driver/shim_check.cpp), linked against
+    the library; without a GPU the program stops at its device check."""
+    import subprocess
+
+    header = open(os.path.join(ROOT, "include", "mcmc_step_hip.h")).read()
+    for name in ("set_dynamic_smem_max_size", "full_smem_size", "leapfrog_max_smem_size", "N_WARP_SAMPLES",
+                 "N_BLKS", "N_BLK_SAMPLES", "N_THREADS", "N_P_ALIGNED", "void mcmc_step("):
+        assert name in header, name
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    exe = tmp_path / "shim_check"
+    cmd = ["g++", "-O1", "-std=c++17", "-Wall", "-Werror", "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(ROOT, "include"),
+           "-I" + os.path.join(rocm, "include"), "-o", str(exe),
+           os.path.join(pkg.PKG_DIR, "driver", "shim_check.cpp"), "-L" + pkg.PKG_DIR, "-lbnn_hmc",
+           "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + pkg.PKG_DIR,
+           "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert r.returncode in (0, 3), r.stdout + r.stderr
+    if r.returncode == 3:
+        assert "no HIP device" in r.stderr
+    # the copy built with the library is there too (the GPU test runs that one)
+    assert os.path.exists(os.path.join(pkg.PKG_DIR, "shim_check"))
+
+
+def test_flag_counter_bound_is_checked_on_the_host(pkg, lib):
+    # the exchange numbers the leapfrog steps of a launch in 32 bits: refused before any device work
+    h = lib.default_hmc(leapfrog_steps=2 ** 30)
+    l = lib.default_launch(transitions_per_launch=8)
+    hnd = C.c_void_p()
+    rc = lib.c.bnnhmc_create(C.byref(lib.default_model()), C.byref(h), C.byref(l), 1, 1, C.byref(hnd))
+    assert rc == pkg.ERR_INVALID and b"2^32" in lib.c.bnnhmc_last_error()

@@ -27,8 +27,9 @@ def say(msg):
 # ------------------------------------------------------------------------------------------------
 @pytest.fixture(scope="module")
 def config0_chain(pkg, lib, orc):
-    """Runs the first 100 transitions (the burn-in) of configs[0] on the GPU, keeps the sampler open
-    for the tests that continue it, and returns what they need."""
+    """Runs the first 100 transitions (the burn-in) of configs[0] on the GPU, one call per transition so
+    that the state every transition started from is on record, keeps the sampler open for the tests that
+    continue it, and returns what they need."""
     model = lib.default_model(n=N_FULL, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
     om = ob.Model(D0, D1, N_FULL, ob.LIK_GAUSSIAN, 0.01, 0.0, 0.1)
     hmc = lib.default_hmc(leapfrog_steps=L_FULL, burn_in=100, n_samples=100, eps0=0.01, seed=0)
@@ -38,8 +39,13 @@ def config0_chain(pkg, lib, orc):
     X, y = s.get_window_data(0)
     s.init_chains(None)
     say("configs[0]: 100 burn-in transitions of 1000 leapfrog steps on the GPU")
-    s.run(100)
-    out = dict(s=s, model=model, om=om, oh=oh, X=X, y=y, traces=s.get_traces(0), state=s.get_chain_state(0))
+    starts = []
+    for t in range(100):
+        st = s.get_chain_state(0)
+        starts.append((np.asarray(st["w"], dtype=np.float32).copy(), np.float32(st["eps"])))
+        s.run(1)
+    out = dict(s=s, model=model, om=om, oh=oh, X=X, y=y, traces=s.get_traces(0), state=s.get_chain_state(0),
+               starts=starts)
     yield out
     s.close()
 
@@ -47,7 +53,8 @@ def config0_chain(pkg, lib, orc):
 def test_first_50_transitions_at_full_size(config0_chain, orc):
     """north-star: identical accept/reject decisions over the first 50 transitions given the same RNG
     stream.  With eps0 = 0.01 this posterior (curvature about n / sigma^2) makes every one of them
-    diverge: all reject, and the step-size trace must equal the oracle's bit for bit."""
+    diverge: all reject, and the step-size trace must equal the oracle's bit for bit.  (The transitions
+    in which accepts and rejects mix come later in the burn-in: next test.)"""
     c = config0_chain
     t0 = time.time()
     ref = orc.run_chain_from(c["om"], c["oh"], c["X"], c["y"], None, 0.01, 0, 50)
@@ -60,6 +67,70 @@ def test_first_50_transitions_at_full_size(config0_chain, orc):
     # the adaptation does arrive: later burn-in transitions accept
     assert tr["accept"][50:100].sum() > 10
     assert 5e-6 < c["state"]["eps"] < 1e-4
+
+
+def test_burn_in_transitions_50_to_100_at_full_size(config0_chain, orc):
+    """The second half of the burn-in of configs[0], where the step size arrives (about transition 65) and
+    accepts and rejects mix: transitions 50 .. 99, each run on the oracle from the very state the GPU
+    started it in (position, step size, RNG counter), as in the adapted leg below.
+
+    Three kinds of transition occur: divergent ones (the step size is still too large: non-finite or
+    hugely negative ratio, below -1000, reject), the first stable ones from the all-zero start (ratios of 1e2 .. 1e6:
+    accept whatever the uniform), and, from about transition 82 on, ratios of order one, where the
+    decision depends on the uniform.  Decisions must agree wherever the uniform is further from the
+    oracle's ratio than the margin 0.3 + 0.1 |log alpha| + 2 |oracle(+1 ulp) - oracle| (the last term, the
+    oracle's own sensitivity to its start, only evaluated where the uniform is within 5 of the ratio);
+    the step size after the transition must be bit-equal wherever the ratio is further than that margin
+    from the adaptation's threshold log 0.2."""
+    c = config0_chain
+    tr, starts = c["traces"], c["starts"]
+    log_target = float(np.log(np.float32(0.2)))
+    n_acc = n_rej_finite = n_div = n_unclear = n_eps_checked = 0
+    t0 = time.time()
+    for t in range(50, 100):
+        w, eps = starts[t]
+        ref = orc.run_chain_from(c["om"], c["oh"], c["X"], c["y"], w, float(eps), t, 1)
+        la_ref, la_gpu = float(ref["log_acpt"][0]), float(tr["log_acpt"][t])
+        lu = orc.log_uniform(0, 0, t)
+        # (an unstable trajectory amplifies every rounding difference: only its verdict is compared; the
+        # uniform is never below log FLT_MIN = -87.3)
+        divergent = (not np.isfinite(la_ref)) or la_ref < -1e3
+        if divergent:
+            assert (not np.isfinite(la_gpu)) or la_gpu < -1e2, (t, la_gpu, la_ref)
+            assert tr["accept"][t] == 0 and ref["accept"][0] == 0
+            assert np.float32(tr["eps"][t]).tobytes() == np.float32(ref["eps"][0]).tobytes(), t
+            n_div += 1
+            continue
+        pert_term = 0.0
+        near = min(abs(lu - la_ref), abs(min(la_ref, 0.0) - log_target))
+        if near < 5.0:
+            w_up = np.nextafter(w, np.float32(np.inf)).astype(np.float32)
+            pert = orc.run_chain_from(c["om"], c["oh"], c["X"], c["y"], w_up, float(eps), t, 1)
+            pert_term = 2.0 * abs(float(pert["log_acpt"][0]) - la_ref)
+        margin = 0.3 + 0.1 * abs(la_ref) + pert_term
+        say("  t=%d eps %.3e log u %.3f log alpha gpu %.6g oracle %.6g margin %.3g accept %d %d" % (
+            t, eps, lu, la_gpu, la_ref, margin, tr["accept"][t], ref["accept"][0]))
+        # the two ratios themselves: same trajectory, same sums
+        assert abs(la_gpu - la_ref) <= 1.0 + 0.2 * abs(la_ref) + pert_term, (t, la_gpu, la_ref)
+        if abs(lu - la_ref) > margin:
+            assert tr["accept"][t] == ref["accept"][0], (t, lu, la_gpu, la_ref)
+        else:
+            n_unclear += 1
+        if abs(min(la_ref, 0.0) - log_target) > margin:
+            assert np.float32(tr["eps"][t]).tobytes() == np.float32(ref["eps"][0]).tobytes(), t
+            n_eps_checked += 1
+        if tr["accept"][t]:
+            n_acc += 1
+        else:
+            n_rej_finite += 1
+    say("transitions 50..99: %d divergent rejects, %d accepts, %d rejects at a finite ratio, %d inside the margin, "
+        "%d step sizes compared bit for bit; oracle time %.0f s" % (
+            n_div, n_acc, n_rej_finite, n_unclear, n_eps_checked + n_div, time.time() - t0))
+    # what this stretch of the chain holds (eps0 = 0.01 needs about 65 decrements before a trajectory is
+    # stable, so the first 90 transitions hold fewer than 15 rejects at a finite ratio; the adapted leg below
+    # adds 20 transitions of which about two thirds reject)
+    assert n_div >= 10 and n_acc >= 20 and n_rej_finite >= 4
+    assert n_unclear <= 8
 
 
 def _log_alpha_f64(orc, X, y, w0, eps, t):
@@ -278,8 +349,8 @@ def test_1600_samples_at_reduced_size(pkg, lib, orc):
 
 
 # ------------------------------------------------------------------------------------------------
-# configs[2] batching: 200 windows of 58368 rows as three batches of 64 (4 workgroups per chain) and
-# a last batch of 8 (widened to 32 workgroups per chain)
+# configs[2] batching: 200 windows of 58368 rows as a batch of 128 (2 workgroups per chain), one of 64
+# (4 per chain) and a last batch of 8 (widened to 32 workgroups per chain)
 # ------------------------------------------------------------------------------------------------
 def test_200_windows_are_batched_without_crosstalk(pkg, lib, orc):
     # a step size small enough that trajectories from the all-zero start are accepted
@@ -396,32 +467,70 @@ def test_single_chain_on_256_workgroups_soak(pkg, lib, orc):
 
 def test_reference_model_first_transitions_at_full_size(pkg, lib, orc):
     """The reference's own model constants (Student-t likelihood, scale 100, 2.2 degrees of freedom, prior scale
-    200: global_params.h:39-48) at full size, from the all-zero start with eps0 = 0.01 as main_loop does
-    (main.h:182-202): the first 12 transitions of 1000 leapfrog steps.  Decisions and the step-size trace must
-    equal the oracle's; this posterior is smooth at that step size (no transition diverges), so the log accept
-    ratios must agree as well, to the rounding noise of their row sums."""
-    say("reference model, 12 transitions of 1000 leapfrog steps at full size")
+    200: global_params.h:39-48) at full size, from the all-zero start as main_loop does (main.h:182-202), 1000
+    leapfrog steps per transition, in two legs.
+    Leg 1, the reference's eps0 = 0.01: the first 50 transitions.  This posterior is smooth at that step size:
+    no transition diverges, the ratios are of order 1e-3 and every proposal is accepted, so decisions and the
+    step-size trace must equal the oracle's, and the log accept ratios must agree to the rounding noise of
+    their row sums.
+    Leg 2, eps0 = 0.25 without adaptation, where the energy error of a trajectory is of order one and accepts
+    and rejects mix: 16 transitions, each restarted on the oracle from the state the GPU started it in;
+    decisions must agree wherever the uniform is further from the oracle's ratio than 0.05 + 0.05 |log alpha|
+    (measured distance between the implementations: see the printed lines)."""
     model = lib.default_model(n=N_FULL)
     om = ob.ref_model(N_FULL)
+    # ---- leg 1 ----
+    n1 = 50
+    say("reference model, %d transitions of 1000 leapfrog steps at full size, eps0 = 0.01" % n1)
     hmc = lib.default_hmc(leapfrog_steps=L_FULL, burn_in=100, n_samples=4, eps0=0.01, seed=0)
     oh = ob.ref_hmc(L_FULL, 100, 4, 0, 0, 0.01)
     s = lib.create(model, hmc, lib.default_launch(), 1, 1)
     s.generate_window(0, teacher_scale=0.1, noise_sigma=0.01)
     X, y = s.get_window_data(0)
     s.init_chains(None)
-    s.run(12)
+    s.run(n1)
     tr = s.get_traces(0)
     s.close()
     t0 = time.time()
-    ref = orc.run_chain_from(om, oh, X, y, None, 0.01, 0, 12)
-    say("oracle: 12 transitions in %.1f s" % (time.time() - t0))
-    assert np.array_equal(tr["accept"][:12], ref["accept"])
-    assert tr["eps"][:12].tobytes() == ref["eps"].tobytes()
+    ref = orc.run_chain_from(om, oh, X, y, None, 0.01, 0, n1)
+    say("oracle: %d transitions in %.1f s" % (n1, time.time() - t0))
+    assert np.array_equal(tr["accept"][:n1], ref["accept"])
+    assert tr["eps"][:n1].tobytes() == ref["eps"].tobytes()
     assert np.all(np.isfinite(ref["log_acpt"]))
-    err = np.abs(tr["log_acpt"][:12].astype(np.float64) - ref["log_acpt"])
+    err = np.abs(tr["log_acpt"][:n1].astype(np.float64) - ref["log_acpt"])
     say("log accept ratios: oracle %s, largest difference %.3g" % (np.array2string(ref["log_acpt"], precision=4),
                                                                   err.max()))
     # the ratios themselves are of order 1e-3 here.  Each is a sum of 58368 differences of per-row
     # log-likelihoods of size 5.6, known to one FP32 ulp (4.8e-7): at random signs that is 1.2e-4 of rounding
-    # noise in either implementation (measured difference: 2.8e-5)
+    # noise in either implementation (measured difference over the first 12: 2.8e-5)
     assert err.max() <= 2e-4
+    # ---- leg 2 ----
+    n2, eps2 = 16, 0.25
+    say("reference model, %d transitions at eps0 = %g, no adaptation" % (n2, eps2))
+    hmc2 = lib.default_hmc(leapfrog_steps=L_FULL, burn_in=0, n_samples=n2, eps0=eps2, seed=0, adapt_steps=0)
+    oh2 = ob.Hmc(L_FULL, 0, n2, 0, eps2, 0.2, 0.1, 0.01, 0, 0)
+    s = lib.create(model, hmc2, lib.default_launch(), 1, 1)
+    s.set_window_data(0, X, y)
+    s.init_chains(None)
+    la_gpu, la_ref, acc_gpu, acc_ref = np.zeros(n2), np.zeros(n2), np.zeros(n2, int), np.zeros(n2, int)
+    t0 = time.time()
+    for k in range(n2):
+        st = s.get_chain_state(0)
+        s.run(1)
+        trk = s.get_traces(0)
+        r = orc.run_chain_from(om, oh2, X, y, np.asarray(st["w"], dtype=np.float32), eps2, k, 1)
+        la_gpu[k], acc_gpu[k] = trk["log_acpt"][k], trk["accept"][k]
+        la_ref[k], acc_ref[k] = r["log_acpt"][0], r["accept"][0]
+    s.close()
+    lu = np.array([orc.log_uniform(0, 0, k) for k in range(n2)])
+    for k in range(n2):
+        say("  t=%d log u %.4f log alpha gpu %.5f oracle %.5f accept %d %d" % (k, lu[k], la_gpu[k], la_ref[k],
+                                                                                acc_gpu[k], acc_ref[k]))
+    say("leg 2: %d of %d accepted (oracle %d), largest |gpu - oracle| %.3g, oracle time %.0f s" % (
+        acc_gpu.sum(), n2, acc_ref.sum(), np.abs(la_gpu - la_ref).max(), time.time() - t0))
+    clear = np.abs(lu - la_ref) > 0.05 + 0.05 * np.abs(la_ref)
+    assert np.all(np.isfinite(la_ref)) and np.all(np.isfinite(la_gpu))
+    assert np.array_equal(acc_gpu[clear], acc_ref[clear])
+    assert clear.sum() >= n2 - 3
+    assert np.all(np.abs(la_gpu - la_ref) <= 0.05 + 0.05 * np.abs(la_ref))
+    assert 3 <= acc_gpu.sum() <= n2 - 3, "the step size was chosen so that accepts and rejects mix"

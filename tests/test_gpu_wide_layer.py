@@ -216,3 +216,35 @@ def test_window_diagnostics_use_the_four_chains(pkg, lib, orc):
     r_host, e_host = lib.split_rhat_ess(chains)
     assert rhat.tobytes() == r_host.tobytes() and ess.tobytes() == e_host.tobytes()
     assert np.all(np.isfinite(rhat)) and np.all(rhat >= 0.5) and np.all(ess > 0)
+
+
+def test_one_transition_at_full_size(pkg, lib, orc):
+    """The scaled shape at its stated size (64 -> 128 -> 1, 233472 rows, 4 workgroups per chain as the
+    batched job runs it): one whole transition of 50 leapfrog steps from the all-zero start with the
+    reference's model constants and eps0 = 0.01, against the oracle: log accept ratio, decision, the state
+    the chain ends in and the step size after adaptation."""
+    n, L = 233472, 50
+    say("64->128->1, one transition of %d leapfrog steps on %d rows" % (L, n))
+    model = lib.default_model(d0=D0, d1=D1, n=n)
+    om = ob.Model(D0, D1, n, ob.LIK_STUDENT_T, 100.0, 2.2, 200.0)
+    hmc = lib.default_hmc(leapfrog_steps=L, burn_in=1, n_samples=1, eps0=0.01, seed=6)
+    s = lib.create(model, hmc, lib.default_launch(cus_per_chain=4), 1, 1)
+    s.generate_window(0, teacher_scale=0.05, noise_sigma=0.01)
+    X, y = s.get_window_data(0)
+    s.init_chains(None)
+    s.run(1)
+    tr, st = s.get_traces(0), s.get_chain_state(0)
+    s.close()
+    ref = orc.run_chain_from(om, ob.Hmc(L, 1, 1, 1, 0.01, 0.2, 0.1, 0.01, 6, 0), X, y, None, 0.01, 0, 1)
+    lu = orc.log_uniform(6, 0, 0)
+    say("log accept ratio: gpu %.6g oracle %.6g, log u %.4f, accepted %d %d" % (
+        tr["log_acpt"][0], ref["log_acpt"][0], lu, tr["accept"][0], ref["accept"][0]))
+    # a sum of 233472 differences of per-row terms of size 5.6, each known to one FP32 ulp (4.8e-7):
+    # 2.3e-4 of rounding noise at random signs in either implementation
+    assert abs(float(tr["log_acpt"][0]) - float(ref["log_acpt"][0])) <= 6e-4
+    assert abs(lu - float(ref["log_acpt"][0])) > 1e-2, "the inputs put the decision on a knife edge"
+    assert tr["accept"][0] == ref["accept"][0] == 1
+    assert np.float32(tr["eps"][0]).tobytes() == np.float32(ref["eps"][0]).tobytes()
+    np.testing.assert_allclose(st["w"], ref["final_w"], rtol=0,
+                               atol=1e-6 * L * max(1.0, float(np.abs(ref["final_w"]).max())))
+    assert float(np.abs(ref["final_w"]).max()) > 0.5         # the chain did move

@@ -7,7 +7,7 @@ import sys
 import numpy as np
 import pytest
 
-from hipmem import DevBuf
+from hipmem import DevBuf, free_bytes, synchronize
 
 pytestmark = pytest.mark.gpu
 
@@ -30,6 +30,14 @@ def _case(pkg, lib, orc, n, L, eps, G, seed, static):
         lib.mcmc_step_static(model, launch, dX.ptr, dy.ptr, dw0.ptr, outs[0].ptr, dm0.ptr, outs[1].ptr, dg0.ptr,
                              outs[2].ptr, outs[3].ptr, dloss.ptr, eps, L, 0)
         lib.step_check(model, launch, 0, 0)
+        # The first call for a configuration has looked up the device, the launch plan and the scratch's
+        # address; a second call only launches kernels: the free device memory is the same before and after
+        synchronize()
+        before = free_bytes()
+        lib.mcmc_step_static(model, launch, dX.ptr, dy.ptr, dw0.ptr, outs[0].ptr, dm0.ptr, outs[1].ptr, dg0.ptr,
+                             outs[2].ptr, outs[3].ptr, dloss.ptr, eps, L, 0)
+        lib.step_check(model, launch, 0, 0)
+        assert free_bytes() == before, "bnnhmc_mcmc_step_static changed the free device memory"
     else:
         wsb = lib.step_workspace_bytes(model, launch)
         ws = DevBuf.full(wsb // 4 + 16, 0, np.int32)
