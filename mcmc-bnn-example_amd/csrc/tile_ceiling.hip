@@ -3,7 +3,9 @@
 // 24 MFMAs 4x4x1), taken from the very header the kernel is built from -- run on registers, with no memory traffic, no barrier and no
 // reduction, two waves per SIMD as in the kernel.  FP32 MFMA and vector instructions share one pipe
 // on this chip, so the time per tile is what that instruction mix costs on it; the production loop can
-// come close to this number but not beat it.  Also times the two halves of the mix alone.
+// come close to this number but not beat it.  Also times the two halves of the mix alone, and two
+// alternative mixes in which the eight hidden units beyond the second 16-wide hidden tile (32 .. 39) leave
+// the half-empty third tile for 4x4x1 blocks (see hybrid_kernel below).
 //
 //   tile_ceiling [tiles per wave]      (default 30000)
 #include <hip/hip_runtime.h>
@@ -86,6 +88,217 @@ __global__ __launch_bounds__(512) void tile_kernel(float* out, unsigned long lon
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Alternative mixes: hidden units 32 .. 39 on v_mfma_f32_4x4x1_16b_f32 (sixteen independent 4x4 blocks).
+//
+// GEMM1, third hidden tile.  Block b = 4 q + cb (lanes 4 b .. 4 b + 3), twelve instructions s = 0 .. 11:
+//     A_b[i] = x_aug[row 4 q + i][k = 12 (cb >> 1) + s]            (lane n = 4 cb + i supplies it)
+//     B_b[r] = W1_aug[k][hidden 32 + 4 (cb & 1) + r]                (lane n = 4 cb + r)
+//     D: lane (n, q), register i: row 4 q + i, hidden 32 + (n & 7), partial over the k-half n >> 3
+//   i.e. the C layout of the 16-wide tiles, except that lanes n >= 8 hold the second half of the
+//   contraction instead of eight padded hidden units: 12 x 8.4 cycles instead of 6 x 32.
+// HYBRID == 1 ("GEMM1 only"): both halves are added into every lane (4 DPP additions, lanes n and n ^ 8 then
+//   hold the same total) and the pointwise stage and GEMM2 go on as in production, whose third tile treats
+//   lanes n >= 8 as padding; the sum of g, which production takes from a padded unit, costs one addition.
+// HYBRID == 2 ("both GEMMs"): lanes n < 8 keep the totals of rows 4 q, 4 q + 1, lanes n >= 8 those of rows
+//   4 q + 2, 4 q + 3 (4 bank-masked DPP additions): the pointwise stage runs on 10 values per lane instead of
+//   12; g is folded into the A operand of GEMM2 (u g: 12 multiplications, none on the rows of x); GEMM2 of
+//   the third tile is 12 blocks instructions  A_b[i] = u g of hidden 32 + 4 (cb & 1) + i, row R = 4 q +
+//   2 (cb >> 1) + rho,  B_b[r] = x_aug[R][feature 6 r + fs]  (fs = 0 .. 5), instead of 4 wide and 8 block
+//   instructions.
+// Both need operands in layouts the production tile does not load: 12 floats per lane and tile for GEMM1
+// (x_aug[row 4 q + (n & 3)][12 (n >> 3) ..+12]) and, for HYBRID == 2, 12 more for GEMM2.  Here they sit in
+// registers: what is timed is the arithmetic alone.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ f4 mfma4(float a, float b, f4 c) { return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ f4 mfma16(float a, float b, f4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+
+template <int HYBRID>
+__global__ __launch_bounds__(512) void hybrid_kernel(float* out, unsigned long long* cycles, int tiles,
+                                                     ModelConsts mc, const float* w) {
+  __shared__ float s_w[Layer::P_AL];
+  for (int p = threadIdx.x; p < Layer::P; p += blockDim.x) s_w[p] = w[p];
+  __syncthreads();
+  const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+  Layer layer;
+  layer.load_weights<1>(s_w, mc);
+  layer.zero_acc();
+  StepCtx cx;
+  cx.n = 1 << 30;
+  cx.ell_prev = nullptr;
+  cx.ell_new = nullptr;
+  Layer::TileIn ti;
+  for (int i = 0; i < Layer::KP; ++i) ti.xa[i] = f2{0.01f * (lane + i), -0.02f * (lane - i)};
+  for (int j = 0; j < 4; ++j) {
+    ti.xe[j] = 0.02f * (n - j);
+    ti.xf[j] = f2{0.03f * (n + j), 0.01f * (q - j)};
+  }
+  ti.y1 = 0.1f * q;
+  float x5a[12], w5[12], x5b[2][6];
+  for (int s = 0; s < 12; ++s) {
+    x5a[s] = 0.01f * (lane - 3 * s);
+    w5[s] = 0.02f * (n + s) - 0.3f;
+    x5b[s / 6][s % 6] = 0.015f * (lane + s);
+  }
+  const float w2g5 = layer.w2g[2];
+  f4 d5[6];
+  for (int fs = 0; fs < 6; ++fs) d5[fs] = f4{0.f, 0.f, 0.f, 0.f};
+  float dw2s5 = 0.0f, gsum = 0.0f;
+  const unsigned long long c0 = __builtin_readcyclecounter();
+  const unsigned long long r0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < tiles; ++it) {
+    asm volatile("" : "+v"(ti.xa[0]), "+v"(ti.xa[1]), "+v"(ti.xa[2]), "+v"(ti.xe[0]), "+v"(ti.xe[1]),
+                      "+v"(ti.xe[2]), "+v"(ti.xe[3]), "+v"(ti.xf[0]), "+v"(ti.xf[1]), "+v"(ti.xf[2]),
+                      "+v"(ti.xf[3]), "+v"(ti.y1));
+    asm volatile("" : "+v"(x5a[0]), "+v"(x5a[1]), "+v"(x5a[2]), "+v"(x5a[3]), "+v"(x5a[4]), "+v"(x5a[5]),
+                      "+v"(x5a[6]), "+v"(x5a[7]), "+v"(x5a[8]), "+v"(x5a[9]), "+v"(x5a[10]), "+v"(x5a[11]));
+    if (HYBRID == 2)
+      asm volatile("" : "+v"(x5b[0][0]), "+v"(x5b[0][1]), "+v"(x5b[0][2]), "+v"(x5b[0][3]), "+v"(x5b[0][4]),
+                        "+v"(x5b[0][5]), "+v"(x5b[1][0]), "+v"(x5b[1][1]), "+v"(x5b[1][2]), "+v"(x5b[1][3]),
+                        "+v"(x5b[1][4]), "+v"(x5b[1][5]));
+    // ---- GEMM1: hidden 0 .. 31 on two 16-wide tiles, hidden 32 .. 39 on 4x4 blocks ----
+    f4 acc[3] = {f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}};
+    // (one block instruction after every wide one: the twelve block instructions accumulate into one register
+    // quadruple and each needs its predecessor's result)
+#pragma unroll
+    for (int i = 0; i < Layer::KP; ++i) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        acc[0] = mfma16(ti.xa[i][h], layer.w1b[2 * i + h][0], acc[0]);
+        acc[2] = mfma4(x5a[4 * i + 2 * h], w5[4 * i + 2 * h], acc[2]);
+        acc[1] = mfma16(ti.xa[i][h], layer.w1b[2 * i + h][1], acc[1]);
+        acc[2] = mfma4(x5a[4 * i + 2 * h + 1], w5[4 * i + 2 * h + 1], acc[2]);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (HYBRID == 1) {
+      // both k-halves into every lane, then the production stages
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[2][j] += dpp_move<0x128>(acc[2][j]);  // row_ror:8
+      float ge[4];
+      f2 gf[4];
+      layer.pointwise<1, false, true>(acc, ti, ge, gf, cx, mc, 0, n, q);
+      gsum += ge[0];  // stands for the one addition that collects the sum of g
+      __builtin_amdgcn_sched_barrier(0);
+      layer.gemm2(acc, ge, gf);
+      __builtin_amdgcn_sched_barrier(0);
+      continue;
+    }
+    // ---- HYBRID == 2 ----
+    // lanes n < 8: rows 4 q, 4 q + 1 (registers 0, 1); lanes n >= 8: rows 4 q + 2, 4 q + 3 (registers 2, 3)
+    float sa = acc[2][2], sb = acc[2][3];
+    asm volatile("s_nop 7\n\t"
+                 "v_add_f32_dpp %[a], %[a], %[a] row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %[b], %[b], %[b] row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %[a], %[p0], %[p0] row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                 "v_add_f32_dpp %[b], %[p1], %[p1] row_ror:8 row_mask:0xf bank_mask:0x3"
+                 : [a] "+v"(sa), [b] "+v"(sb)
+                 : [p0] "v"(acc[2][0]), [p1] "v"(acc[2][1]));
+    float yh[4] = {layer.y_0, layer.y_0, layer.y_0, layer.y_0};
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float e = __builtin_amdgcn_exp2f(acc[t][j]);
+        const float sg = __builtin_amdgcn_rcpf(1.0f + e);
+        acc[t][j] = sg;
+        yh[j] = __builtin_fmaf(layer.w2g[t], sg, yh[j]);
+      }
+    }
+    sa = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(sa));
+    sb = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(sb));
+    // the third tile's terms of the row sums: each lane holds two of its four rows
+    asm volatile("s_nop 1\n\t"
+                 "v_fmac_f32_dpp %[y0], %[a], %[w] quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0x3\n\t"
+                 "v_fmac_f32_dpp %[y2], %[a], %[w] quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xc\n\t"
+                 "v_fmac_f32_dpp %[y1], %[b], %[w] quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0x3\n\t"
+                 "v_fmac_f32_dpp %[y3], %[b], %[w] quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xc"
+                 : [y0] "+v"(yh[0]), [y1] "+v"(yh[1]), [y2] "+v"(yh[2]), [y3] "+v"(yh[3])
+                 : [a] "v"(sa), [b] "v"(sb), [w] "v"(w2g5));
+    const float gz = row16_reduce4(yh[0], yh[1], yh[2], yh[3]) + __builtin_fmaf(ti.y1, layer.k2v, layer.rho);
+    gsum += gz;
+    // dw2s += g s  and  u g = (s - s^2) g, g of row 4 q + j read from bank j of gz
+    float ug[2][4], uga, ugb;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ug[t][j] = __builtin_fmaf(-acc[t][j], acc[t][j], acc[t][j]);
+    }
+    uga = __builtin_fmaf(-sa, sa, sa);
+    ugb = __builtin_fmaf(-sb, sb, sb);
+#define BNN_BC(j) " row_newbcast:" #j " row_mask:0xf bank_mask:0xf\n\t"
+    asm volatile("s_nop 1\n\t"
+                 "v_fmac_f32_dpp %[d0], %[g], %[s00]" BNN_BC(0)
+                 "v_fmac_f32_dpp %[d1], %[g], %[s10]" BNN_BC(0)
+                 "v_fmac_f32_dpp %[d0], %[g], %[s01]" BNN_BC(4)
+                 "v_fmac_f32_dpp %[d1], %[g], %[s11]" BNN_BC(4)
+                 "v_fmac_f32_dpp %[d0], %[g], %[s02]" BNN_BC(8)
+                 "v_fmac_f32_dpp %[d1], %[g], %[s12]" BNN_BC(8)
+                 "v_fmac_f32_dpp %[d0], %[g], %[s03]" BNN_BC(12)
+                 "v_fmac_f32_dpp %[d1], %[g], %[s13]" BNN_BC(12)
+                 "v_fmac_f32_dpp %[d5], %[g], %[sa] row_newbcast:0 row_mask:0xf bank_mask:0x3\n\t"
+                 "v_fmac_f32_dpp %[d5], %[g], %[sa] row_newbcast:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_fmac_f32_dpp %[d5], %[g], %[sb] row_newbcast:4 row_mask:0xf bank_mask:0x3\n\t"
+                 "v_fmac_f32_dpp %[d5], %[g], %[sb] row_newbcast:12 row_mask:0xf bank_mask:0xc"
+                 : [d0] "+v"(layer.dw2s[0]), [d1] "+v"(layer.dw2s[1]), [d5] "+v"(dw2s5)
+                 : [g] "v"(gz), [s00] "v"(acc[0][0]), [s01] "v"(acc[0][1]), [s02] "v"(acc[0][2]), [s03] "v"(acc[0][3]),
+                   [s10] "v"(acc[1][0]), [s11] "v"(acc[1][1]), [s12] "v"(acc[1][2]), [s13] "v"(acc[1][3]),
+                   [sa] "v"(sa), [sb] "v"(sb));
+    asm volatile("s_nop 1\n\t"
+                 "v_mul_f32_dpp %[u00], %[g], %[u00]" BNN_BC(0)
+                 "v_mul_f32_dpp %[u10], %[g], %[u10]" BNN_BC(0)
+                 "v_mul_f32_dpp %[u01], %[g], %[u01]" BNN_BC(4)
+                 "v_mul_f32_dpp %[u11], %[g], %[u11]" BNN_BC(4)
+                 "v_mul_f32_dpp %[u02], %[g], %[u02]" BNN_BC(8)
+                 "v_mul_f32_dpp %[u12], %[g], %[u12]" BNN_BC(8)
+                 "v_mul_f32_dpp %[u03], %[g], %[u03]" BNN_BC(12)
+                 "v_mul_f32_dpp %[u13], %[g], %[u13]" BNN_BC(12)
+                 "v_mul_f32_dpp %[ua], %[g], %[ua] row_newbcast:0 row_mask:0xf bank_mask:0x3\n\t"
+                 "v_mul_f32_dpp %[ua], %[g], %[ua] row_newbcast:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_mul_f32_dpp %[ub], %[g], %[ub] row_newbcast:4 row_mask:0xf bank_mask:0x3\n\t"
+                 "v_mul_f32_dpp %[ub], %[g], %[ub] row_newbcast:12 row_mask:0xf bank_mask:0xc"
+                 : [u00] "+v"(ug[0][0]), [u01] "+v"(ug[0][1]), [u02] "+v"(ug[0][2]), [u03] "+v"(ug[0][3]),
+                   [u10] "+v"(ug[1][0]), [u11] "+v"(ug[1][1]), [u12] "+v"(ug[1][2]), [u13] "+v"(ug[1][3]),
+                   [ua] "+v"(uga), [ub] "+v"(ugb)
+                 : [g] "v"(gz));
+#undef BNN_BC
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- GEMM2: hidden 0 .. 31 as in production (g now rides on A), hidden 32 .. 39 on 4x4 blocks ----
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      layer.dacc_e[0] = mfma16(ug[0][j], ti.xe[j], layer.dacc_e[0]);
+      layer.dacc_e[1] = mfma16(ug[1][j], ti.xe[j], layer.dacc_e[1]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        layer.dacc_f[t][0] = mfma4(ug[t][j], ti.xf[j][0], layer.dacc_f[t][0]);
+        layer.dacc_f[t][1] = mfma4(ug[t][j], ti.xf[j][1], layer.dacc_f[t][1]);
+      }
+    }
+#pragma unroll
+    for (int fs = 0; fs < 6; ++fs) {
+      d5[fs] = mfma4(uga, x5b[0][fs], d5[fs]);
+      d5[fs] = mfma4(ugb, x5b[1][fs], d5[fs]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  const unsigned long long c1 = __builtin_readcyclecounter();
+  float sum = dw2s5 + gsum;
+  for (int fs = 0; fs < 6; ++fs)
+    for (int j = 0; j < 4; ++j) sum += d5[fs][j];
+  for (int t = 0; t < Layer::NT; ++t) {
+    sum += layer.dw2s[t];
+    for (int j = 0; j < 4; ++j) sum += layer.dacc_e[t][j] + layer.dacc_f[t][0][j] + layer.dacc_f[t][1][j];
+  }
+  out[blockIdx.x * blockDim.x + threadIdx.x] = sum;
+  if (threadIdx.x == 0) {
+    cycles[2 * blockIdx.x] = c1 - c0;
+    cycles[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+}
+
 #define HIP_CHECK(x)                                                                    \
   do {                                                                                  \
     hipError_t e_ = (x);                                                                \
@@ -95,18 +308,18 @@ __global__ __launch_bounds__(512) void tile_kernel(float* out, unsigned long lon
     }                                                                                   \
   } while (0)
 
-template <int MODE>
-int run(const char* what, int tiles, float* d_out, unsigned long long* d_cyc, const ModelConsts& mc,
-        const float* d_w) {
+typedef void (*TileKernel)(float*, unsigned long long*, int, ModelConsts, const float*);
+int run(TileKernel kernel, const char* what, int tiles, float* d_out, unsigned long long* d_cyc,
+        const ModelConsts& mc, const float* d_w) {
   const int wgs = 256;
   hipEvent_t e0, e1;
   HIP_CHECK(hipEventCreate(&e0));
   HIP_CHECK(hipEventCreate(&e1));
   // warm-up long enough for the clocks to settle
-  hipLaunchKernelGGL(tile_kernel<MODE>, dim3(wgs), dim3(512), 0, 0, d_out, d_cyc, 10 * tiles, mc, d_w);
+  hipLaunchKernelGGL(kernel, dim3(wgs), dim3(512), 0, 0, d_out, d_cyc, 10 * tiles, mc, d_w);
   HIP_CHECK(hipDeviceSynchronize());
   HIP_CHECK(hipEventRecord(e0));
-  hipLaunchKernelGGL(tile_kernel<MODE>, dim3(wgs), dim3(512), 0, 0, d_out, d_cyc, tiles, mc, d_w);
+  hipLaunchKernelGGL(kernel, dim3(wgs), dim3(512), 0, 0, d_out, d_cyc, tiles, mc, d_w);
   HIP_CHECK(hipEventRecord(e1));
   HIP_CHECK(hipEventSynchronize(e1));
   float ms = 0;
@@ -145,8 +358,10 @@ int main(int argc, char** argv) {
   HIP_CHECK(hipMemcpy(d_w, w.data(), w.size() * sizeof(float), hipMemcpyHostToDevice));
   std::printf("tile of 16 rows, 22 -> 40 -> 1, two waves per SIMD, %d tiles per wave, 256 workgroups of 512 threads\n",
               tiles);
-  if (run<0>("whole tile (MFMAs + pointwise)", tiles, d_out, d_cyc, mc, d_w)) return 1;
-  if (run<1>("the MFMAs alone", tiles, d_out, d_cyc, mc, d_w)) return 1;
-  if (run<2>("the pointwise stage alone", tiles, d_out, d_cyc, mc, d_w)) return 1;
+  if (run(tile_kernel<0>, "whole tile (MFMAs + pointwise)", tiles, d_out, d_cyc, mc, d_w)) return 1;
+  if (run(tile_kernel<1>, "the MFMAs alone", tiles, d_out, d_cyc, mc, d_w)) return 1;
+  if (run(tile_kernel<2>, "the pointwise stage alone", tiles, d_out, d_cyc, mc, d_w)) return 1;
+  if (run(hybrid_kernel<1>, "hidden 32..39 on 4x4 blocks: GEMM1", tiles, d_out, d_cyc, mc, d_w)) return 1;
+  if (run(hybrid_kernel<2>, "hidden 32..39 on 4x4 blocks: both", tiles, d_out, d_cyc, mc, d_w)) return 1;
   return 0;
 }

@@ -85,7 +85,7 @@ def test_burn_in_transitions_50_to_100_at_full_size(config0_chain, orc):
     c = config0_chain
     tr, starts = c["traces"], c["starts"]
     log_target = float(np.log(np.float32(0.2)))
-    n_acc = n_rej_finite = n_div = n_unclear = n_eps_checked = 0
+    n_acc = n_rej_finite = n_div = n_unclear = n_eps_checked = n_big = 0
     t0 = time.time()
     for t in range(50, 100):
         w, eps = starts[t]
@@ -100,6 +100,16 @@ def test_burn_in_transitions_50_to_100_at_full_size(config0_chain, orc):
             assert tr["accept"][t] == 0 and ref["accept"][0] == 0
             assert np.float32(tr["eps"][t]).tobytes() == np.float32(ref["eps"][0]).tobytes(), t
             n_div += 1
+            continue
+        if la_ref > 100.0:
+            # the first stable trajectories from the all-zero start, just inside the stability limit of the
+            # integrator: ratios of 1e2 .. 1e6 that differ by tens of percent between implementations (and
+            # between two oracle runs one ulp apart); accepted whatever the uniform, step size incremented
+            say("  t=%d eps %.3e log alpha gpu %.6g oracle %.6g: accept whatever the uniform" % (t, eps, la_gpu, la_ref))
+            assert la_gpu > 10.0 and tr["accept"][t] == 1 and ref["accept"][0] == 1, (t, la_gpu, la_ref)
+            assert np.float32(tr["eps"][t]).tobytes() == np.float32(ref["eps"][0]).tobytes(), t
+            n_acc += 1
+            n_big += 1
             continue
         pert_term = 0.0
         near = min(abs(lu - la_ref), abs(min(la_ref, 0.0) - log_target))
@@ -123,13 +133,13 @@ def test_burn_in_transitions_50_to_100_at_full_size(config0_chain, orc):
             n_acc += 1
         else:
             n_rej_finite += 1
-    say("transitions 50..99: %d divergent rejects, %d accepts, %d rejects at a finite ratio, %d inside the margin, "
-        "%d step sizes compared bit for bit; oracle time %.0f s" % (
-            n_div, n_acc, n_rej_finite, n_unclear, n_eps_checked + n_div, time.time() - t0))
+    say("transitions 50..99: %d divergent rejects, %d accepts (%d of them at ratios above 100), %d rejects at a "
+        "finite ratio, %d inside the margin, %d step sizes compared bit for bit; oracle time %.0f s" % (
+            n_div, n_acc, n_big, n_rej_finite, n_unclear, n_eps_checked + n_div + n_big, time.time() - t0))
     # what this stretch of the chain holds (eps0 = 0.01 needs about 65 decrements before a trajectory is
     # stable, so the first 90 transitions hold fewer than 15 rejects at a finite ratio; the adapted leg below
     # adds 20 transitions of which about two thirds reject)
-    assert n_div >= 10 and n_acc >= 20 and n_rej_finite >= 4
+    assert n_div >= 10 and n_acc >= 20 and n_acc - n_big >= 8 and n_rej_finite >= 4
     assert n_unclear <= 8
 
 
@@ -183,7 +193,7 @@ def test_20_transitions_from_the_adapted_state_at_full_size(config0_chain, orc):
     how far the GPU is from it (0.113), while a float64 trajectory lies between them (GPU 0.06 from
     it, oracle 0.09).  So the bounds are stated against that sensitivity, measured in the test:
       a. rms |GPU - oracle| over the 20 transitions <= 2 rms |oracle(+1 ulp) - oracle| + 0.02;
-      b. over the first 6 transitions, rms |GPU - float64| <= 2.5 rms |oracle - float64| + 0.03;
+      b. over the first 4 transitions, rms |GPU - float64| <= 2.5 rms |oracle - float64| + 0.03;
       c. no transition differs by more than 1 + 0.2 |log alpha| (a missing term or row range);
       d. decisions agree wherever the uniform is further from the oracle's ratio than the margin
          0.3 + 0.1 |log alpha| + 2 |oracle(+1 ulp) - oracle|; at least 10 of the 20 are that clear,
@@ -192,7 +202,7 @@ def test_20_transitions_from_the_adapted_state_at_full_size(config0_chain, orc):
     s = c["s"]
     assert c["state"]["transitions_done"] == 100
     eps_adapted = np.float32(c["state"]["eps"])
-    n_tr, n_f64 = 20, 6
+    n_tr, n_f64 = 20, 4
     la_gpu, la_ref, la_pert, la_f64 = np.zeros(n_tr), np.zeros(n_tr), np.zeros(n_tr), np.zeros(n_f64)
     acc_gpu, acc_ref = np.zeros(n_tr, dtype=np.int64), np.zeros(n_tr, dtype=np.int64)
     t0 = time.time()
@@ -474,9 +484,9 @@ def test_reference_model_first_transitions_at_full_size(pkg, lib, orc):
     step-size trace must equal the oracle's, and the log accept ratios must agree to the rounding noise of
     their row sums.
     Leg 2, eps0 = 0.25 without adaptation, where the energy error of a trajectory is of order one and accepts
-    and rejects mix: 16 transitions, each restarted on the oracle from the state the GPU started it in;
-    decisions must agree wherever the uniform is further from the oracle's ratio than 0.05 + 0.05 |log alpha|
-    (measured distance between the implementations: see the printed lines)."""
+    and rejects mix: 14 transitions, each restarted on the oracle from the state the GPU started it in.  The
+    ratios (of order one) must agree within 2e-3 + 1e-3 |log alpha| (measured: 2.1e-4 at most), and decisions
+    wherever the uniform is further from the oracle's ratio than that."""
     model = lib.default_model(n=N_FULL)
     om = ob.ref_model(N_FULL)
     # ---- leg 1 ----
@@ -505,7 +515,7 @@ def test_reference_model_first_transitions_at_full_size(pkg, lib, orc):
     # noise in either implementation (measured difference over the first 12: 2.8e-5)
     assert err.max() <= 2e-4
     # ---- leg 2 ----
-    n2, eps2 = 16, 0.25
+    n2, eps2 = 14, 0.25
     say("reference model, %d transitions at eps0 = %g, no adaptation" % (n2, eps2))
     hmc2 = lib.default_hmc(leapfrog_steps=L_FULL, burn_in=0, n_samples=n2, eps0=eps2, seed=0, adapt_steps=0)
     oh2 = ob.Hmc(L_FULL, 0, n2, 0, eps2, 0.2, 0.1, 0.01, 0, 0)
@@ -528,9 +538,10 @@ def test_reference_model_first_transitions_at_full_size(pkg, lib, orc):
                                                                                 acc_gpu[k], acc_ref[k]))
     say("leg 2: %d of %d accepted (oracle %d), largest |gpu - oracle| %.3g, oracle time %.0f s" % (
         acc_gpu.sum(), n2, acc_ref.sum(), np.abs(la_gpu - la_ref).max(), time.time() - t0))
-    clear = np.abs(lu - la_ref) > 0.05 + 0.05 * np.abs(la_ref)
+    tol = 2e-3 + 1e-3 * np.abs(la_ref)
+    clear = np.abs(lu - la_ref) > tol
     assert np.all(np.isfinite(la_ref)) and np.all(np.isfinite(la_gpu))
     assert np.array_equal(acc_gpu[clear], acc_ref[clear])
-    assert clear.sum() >= n2 - 3
-    assert np.all(np.abs(la_gpu - la_ref) <= 0.05 + 0.05 * np.abs(la_ref))
+    assert clear.sum() >= n2 - 1
+    assert np.all(np.abs(la_gpu - la_ref) <= tol)
     assert 3 <= acc_gpu.sum() <= n2 - 3, "the step size was chosen so that accepts and rejects mix"
