@@ -10,7 +10,7 @@ the same assembly statement, so the kernels that use only those may spill freely
 import re
 import sys
 
-ASM_LOAD_KERNELS = ("MfmaLayerILi22ELi40ELi2EEE", "hmc_kernel_wide")
+ASM_LOAD_KERNELS = ("MfmaLayerILi22ELi40ELi2EEE", "MfmaHybridLayer", "hmc_kernel_wide")
 
 
 def main(path):

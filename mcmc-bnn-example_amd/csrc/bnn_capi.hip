@@ -123,6 +123,12 @@ int query_device(DeviceInfo& di) {
   return BNNHMC_OK;
 }
 
+// Measurement switch: BNNHMC_PIPELINE=<n> selects the MFMA tile loop of launches that leave `pipeline` at
+// its default (and the thread count at 512).  Unset in normal use.
+int env_pipeline() {
+  const char* e = getenv("BNNHMC_PIPELINE");
+  return e && *e ? atoi(e) : 0;
+}
 // How a launch is laid over the GPU
 struct Plan {
   const void* kernel = nullptr;
@@ -157,7 +163,7 @@ int make_plan_uncached(const bnnhmc_model& m, const bnnhmc_launch* lp, const Dev
     return fail(BNNHMC_ERR_INVALID, "wgs_per_cu must be 1 or 2, got %d", l.wgs_per_cu);
   // MFMA tile loop: 0 / 2 = explicitly prefetched loop (default), 1 = software-pipelined, 3 = plain
   int loop = 0;
-  if (l.layer == BNNHMC_LAYER_MFMA) loop = l.pipeline == 1 ? 1 : (l.pipeline == 3 ? 0 : 2);
+  if (l.layer == BNNHMC_LAYER_MFMA) loop = l.pipeline == 1 ? 1 : (l.pipeline == 3 ? 0 : (l.pipeline == 4 ? 4 : 2));
   // the prefetched loop exists for 512 threads only; other sizes get the plain loop unless the
   // prefetched one was asked for by name (then there is no kernel, reported below)
   if (l.layer == BNNHMC_LAYER_MFMA && l.pipeline == 0 && l.threads > 0 && l.threads != 512) loop = 0;
@@ -173,6 +179,8 @@ int make_plan_uncached(const bnnhmc_model& m, const bnnhmc_launch* lp, const Dev
   } else {
     p.threads = l.threads > 0 ? l.threads
                               : (l.layer == BNNHMC_LAYER_FFMA || l.wgs_per_cu == 2 ? 256 : 512);
+    if (l.layer == BNNHMC_LAYER_MFMA && l.pipeline == 0 && p.threads == 512 && env_pipeline() > 0)
+      loop = env_pipeline() == 3 ? 0 : env_pipeline();
     p.kernel = hmc_kernel_for(m.d0, m.d1, l.layer, m.lik_kind, p.threads, loop);
   }
   if (!p.kernel)

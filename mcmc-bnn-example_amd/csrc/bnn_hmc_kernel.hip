@@ -19,6 +19,7 @@
 #include "bnn_device.h"
 #include "bnn_kernel_common.h"
 #include "bnn_kernels.h"
+#include "bnn_mfma_hybrid_layer.h"
 #include "bnn_mfma_layer.h"
 #include "bnn_rng.h"
 
@@ -39,6 +40,7 @@ struct FfmaLayer {
   static constexpr int HU = D1 / 8;
   static constexpr int oB1 = D0 * D1, oW2 = oB1 + D1, oB2 = oW2 + D1, P = oB2 + 1;
   static constexpr int P_AL = (P + 3) / 4 * 4;
+  static constexpr int TILE_LDS = 0;  // no copy of the tile in LDS
 
   float w1[D0][HU];
   float b1[HU];
@@ -235,6 +237,8 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   __shared__ double s_red[W];
   __shared__ unsigned long long s_hash[W];
   __shared__ int s_progress[W];
+  // a wave's copy of the tile it is working on (the hybrid MFMA layer only)
+  __shared__ __align__(16) float s_tile[W][Layer::TILE_LDS > 0 ? Layer::TILE_LDS : 4];
   // kept out of registers while a trajectory runs (a thread only ever touches the entries of the
   // parameters it owns, so no barrier guards them): the accepted position and its gradient, the
   // start momentum of the running transition, and the thread's state hash
@@ -286,6 +290,7 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   cx.progress = (a.balance && W == 8) ? s_progress : nullptr;
   cx.wave = wave;
   cx.partner = wave ^ (W / 2);
+  cx.tile_lds = s_tile[wave];
 
   const ModelConsts mc = a.mc;
   // records of flagged packets (8 bytes per parameter), two per workgroup (by step parity)
@@ -772,8 +777,12 @@ const void* hmc_kernel_for(int d0, int d1, int layer, int lik, int threads, int 
   using MP = MfmaLayer<22, 40, 1>;
   using MS = MfmaLayer<22, 40, 0>;
   using MA = MfmaLayer<22, 40, 2>;
+  using MH = MfmaHybridLayer<22, 40>;
   using F = FfmaLayer<22, 40>;
-  if (layer == 0 && pipeline == 2) {
+  if (layer == 0 && pipeline == 4) {
+    // hidden units 32 .. 39 on 4x4 blocks (bnn_mfma_hybrid_layer.h): prefetched loop, 512 threads only
+    if (threads == 512) return lik == 0 ? kernel_ptr<MH, 0, 512>() : kernel_ptr<MH, 1, 512>();
+  } else if (layer == 0 && pipeline == 2) {
     // The prefetched loop is built for 512 threads only.  Its loads are issued from inline assembly
     // and land in their registers long after the compiler believes them written: with fewer than
     // 256 VGPRs per thread (768 or 1024 threads) the kernel spills, and a register that is spilled or

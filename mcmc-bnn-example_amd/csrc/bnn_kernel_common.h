@@ -263,6 +263,7 @@ struct StepCtx {
   float* ell_new;         // last step only: where to store this state's rows (null = skip)
   int* progress;          // LDS, one word per wave: tiles done in this step (null = no balancing)
   int wave, partner;      // this wave and the wave it shares a SIMD with
+  float* tile_lds;        // LDS, this wave's copy of the tile it is working on (layers that keep one)
 };
 
 // ------------------------------------------------------------------------------------------------

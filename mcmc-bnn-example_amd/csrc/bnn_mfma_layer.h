@@ -63,6 +63,7 @@ struct MfmaLayer {
   static_assert(D0 > 16 && D0 + 2 <= 24, "features 16 .. D0 + 1 go through the 4x4 blocks");
   static constexpr int oB1 = D0 * D1, oW2 = oB1 + D1, oB2 = oW2 + D1, P = oB2 + 1;
   static constexpr int P_AL = (P + 3) / 4 * 4;
+  static constexpr int TILE_LDS = 0;  // no copy of the tile in LDS
 
   // The activation is carried as the logistic value s = 1 / (1 + 2^t) = (h + 1) / 2 and h = tanh is
   // never formed: the layer-2 dot, the layer-2 weight gradient and 1 - h^2 = 4 s (1 - s) are all

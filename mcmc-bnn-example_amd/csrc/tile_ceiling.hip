@@ -5,9 +5,11 @@
 // on this chip, so the time per tile is what that instruction mix costs on it; the production loop can
 // come close to this number but not beat it.  Also times the two halves of the mix alone, and two
 // alternative mixes in which the eight hidden units beyond the second 16-wide hidden tile (32 .. 39) leave
-// the half-empty third tile for 4x4x1 blocks (see hybrid_kernel below).
+// the half-empty third tile for 4x4x1 blocks (see hybrid_kernel below).  Then the same for the tile of the
+// 64 -> 128 -> 1 kernel (256 v_mfma_f32_16x16x4_f32 per 16-row tile, the W1 operand read from LDS, one wave
+// per SIMD as in that kernel): whole tile, matrix instructions alone, pointwise stage alone.
 //
-//   tile_ceiling [tiles per wave]      (default 30000)
+//   tile_ceiling [tiles per wave]      (default 30000; the 64 -> 128 -> 1 tile runs a fifth of them)
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
@@ -15,6 +17,7 @@
 #include <vector>
 
 #include "bnn_mfma_layer.h"
+#include "bnn_mfma_wide_layer.h"
 
 using namespace bnn;
 using Layer = MfmaLayer<22, 40, 2>;
@@ -299,6 +302,60 @@ __global__ __launch_bounds__(512) void hybrid_kernel(float* out, unsigned long l
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The tile of the 64 -> 128 -> 1 kernel: MfmaWideLayer::compute_tile on a tile held in registers, the
+// weights in LDS as in the kernel, 256 threads per workgroup = one wave per SIMD.
+// ------------------------------------------------------------------------------------------------
+// Two tiles per trip with nothing between them, as in the kernel's loop (the compiler may overlap the end
+// of one tile with the start of the next).
+using WideLayer = MfmaWideLayer<64, 128>;
+template <int PARTS>
+__global__ __launch_bounds__(256) void wide_kernel(float* out, unsigned long long* cycles, int tiles,
+                                                   ModelConsts mc, const float* w) {
+  __shared__ __align__(16) float s_w[WideLayer::P_AL];
+  for (int p = threadIdx.x; p < WideLayer::P; p += blockDim.x) s_w[p] = w[p % Layer::P];
+  __syncthreads();
+  const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+  WideLayer layer;
+  layer.prepare_step(s_w, mc);
+  layer.zero_acc();
+  StepCtx cx;
+  cx.n = 1 << 30;
+  cx.ell_prev = nullptr;
+  cx.ell_new = nullptr;
+  WideLayer::Tile ti;
+  for (int i = 0; i < WideLayer::KQ; ++i) ti.xa[i] = f4{0.01f * (lane + i), -0.02f * (lane - i), 0.03f * i, 0.01f * q};
+  for (int j = 0; j < 4; ++j)
+    for (int v = 0; v < WideLayer::FV; ++v) ti.xb[j][v] = f2{0.03f * (n + j), 0.01f * (q - j + v)};
+  ti.y1 = 0.1f * q;
+  const unsigned long long c0 = __builtin_readcyclecounter();
+  const unsigned long long r0 = __builtin_amdgcn_s_memrealtime();
+  WideLayer::Tile tj = ti;
+  auto opaque = [](WideLayer::Tile& t) {
+    asm volatile("" : "+v"(t.xa[0]), "+v"(t.xa[1]), "+v"(t.xa[2]), "+v"(t.xa[3]), "+v"(t.xb[0][0]),
+                      "+v"(t.xb[0][1]), "+v"(t.xb[1][0]), "+v"(t.xb[1][1]), "+v"(t.xb[2][0]),
+                      "+v"(t.xb[2][1]), "+v"(t.xb[3][0]), "+v"(t.xb[3][1]), "+v"(t.y1));
+  };
+  for (int it = 0; it < tiles; it += 2) {
+    opaque(ti);
+    opaque(tj);
+    layer.compute_tile<1, false, true, PARTS>(ti, s_w, cx, mc, 0, n, q);
+    layer.compute_tile<1, false, true, PARTS>(tj, s_w, cx, mc, 16, n, q);
+  }
+  const unsigned long long c1 = __builtin_readcyclecounter();
+  float sum = layer.db2acc;
+  for (int t = 0; t < WideLayer::NT; ++t) {
+    sum += layer.dw2acc[t] + layer.db1acc[t];
+    for (int ft = 0; ft < WideLayer::FT; ++ft)
+      for (int j = 0; j < 4; ++j) sum += layer.dacc[t][ft][j];
+  }
+  out[blockIdx.x * blockDim.x + threadIdx.x] = sum;
+  if (threadIdx.x == 0) {
+    cycles[2 * blockIdx.x] = c1 - c0;
+    cycles[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+}
+
 #define HIP_CHECK(x)                                                                    \
   do {                                                                                  \
     hipError_t e_ = (x);                                                                \
@@ -310,16 +367,16 @@ __global__ __launch_bounds__(512) void hybrid_kernel(float* out, unsigned long l
 
 typedef void (*TileKernel)(float*, unsigned long long*, int, ModelConsts, const float*);
 int run(TileKernel kernel, const char* what, int tiles, float* d_out, unsigned long long* d_cyc,
-        const ModelConsts& mc, const float* d_w) {
+        const ModelConsts& mc, const float* d_w, int threads = 512) {
   const int wgs = 256;
   hipEvent_t e0, e1;
   HIP_CHECK(hipEventCreate(&e0));
   HIP_CHECK(hipEventCreate(&e1));
   // warm-up long enough for the clocks to settle
-  hipLaunchKernelGGL(kernel, dim3(wgs), dim3(512), 0, 0, d_out, d_cyc, 10 * tiles, mc, d_w);
+  hipLaunchKernelGGL(kernel, dim3(wgs), dim3(threads), 0, 0, d_out, d_cyc, 10 * tiles, mc, d_w);
   HIP_CHECK(hipDeviceSynchronize());
   HIP_CHECK(hipEventRecord(e0));
-  hipLaunchKernelGGL(kernel, dim3(wgs), dim3(512), 0, 0, d_out, d_cyc, tiles, mc, d_w);
+  hipLaunchKernelGGL(kernel, dim3(wgs), dim3(threads), 0, 0, d_out, d_cyc, tiles, mc, d_w);
   HIP_CHECK(hipEventRecord(e1));
   HIP_CHECK(hipEventSynchronize(e1));
   float ms = 0;
@@ -331,12 +388,12 @@ int run(TileKernel kernel, const char* what, int tiles, float* d_out, unsigned l
     mean += (double)cyc[2 * i] / wgs;
     real += (double)cyc[2 * i + 1] / wgs;
   }
-  // A SIMD holds two waves and issues the older one first, so a wave's own start-to-end ticks say little;
-  // the launch as a whole takes 2 * tiles tiles per SIMD, and the shader clock is the ratio of the two
-  // counters that one wave read.
+  // A SIMD holds threads / 256 waves (two in the 22 -> 40 -> 1 kernel, where it issues the older one first,
+  // so a wave's own start-to-end ticks say little); the launch as a whole takes that many times `tiles` tiles
+  // per SIMD, and the shader clock is the ratio of the two counters that one wave read.
   const double mhz = mean / (real * 1e-2);
-  std::printf("%-34s %9.3f ms (events), shader clock %.0f MHz, %8.1f cycles per tile and SIMD\n", what, ms, mhz,
-              ms * 1e-3 * mhz * 1e6 / (2.0 * tiles));
+  std::printf("%-36s %9.3f ms (events), shader clock %.0f MHz, %8.1f cycles per tile and SIMD\n", what, ms, mhz,
+              ms * 1e-3 * mhz * 1e6 / ((threads / 256) * (double)tiles));
   return 0;
 }
 
@@ -363,5 +420,10 @@ int main(int argc, char** argv) {
   if (run(tile_kernel<2>, "the pointwise stage alone", tiles, d_out, d_cyc, mc, d_w)) return 1;
   if (run(hybrid_kernel<1>, "hidden 32..39 on 4x4 blocks: GEMM1", tiles, d_out, d_cyc, mc, d_w)) return 1;
   if (run(hybrid_kernel<2>, "hidden 32..39 on 4x4 blocks: both", tiles, d_out, d_cyc, mc, d_w)) return 1;
+  const int wt = tiles / 5 > 0 ? tiles / 5 : 1;
+  std::printf("tile of 16 rows, 64 -> 128 -> 1, one wave per SIMD, %d tiles per wave, 256 workgroups of 256 threads\n", wt);
+  if (run(wide_kernel<3>, "whole tile (MFMAs + pointwise)", wt, d_out, d_cyc, mc, d_w, 256)) return 1;
+  if (run(wide_kernel<1>, "the MFMAs and their LDS operand reads", wt, d_out, d_cyc, mc, d_w, 256)) return 1;
+  if (run(wide_kernel<2>, "the pointwise stage alone", wt, d_out, d_cyc, mc, d_w, 256)) return 1;
   return 0;
 }
