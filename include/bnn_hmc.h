@@ -70,7 +70,7 @@ typedef struct bnnhmc_hmc {
 
 /* How the work is laid over the GPU.  Zero in a field selects the default. */
 typedef struct bnnhmc_launch {
-  int layer;          /* BNNHMC_LAYER_MFMA (v_mfma_f32_16x16x4_f32) or BNNHMC_LAYER_FFMA          */
+  int layer;          /* BNNHMC_LAYER_MFMA (v_mfma_f32_16x16x4_f32, _4x4x1_16b_f32) or BNNHMC_LAYER_FFMA */
   int cus_per_chain;  /* workgroups that share one chain's rows; 0 = automatic.  Sampler,         */
                       /* 22 -> 40 -> 1: a batch is the largest power-of-two number of chains that */
                       /* fits, spread over the whole device (one chain: 256 workgroups; 128 or     */
@@ -86,9 +86,11 @@ typedef struct bnnhmc_launch {
                       /* FFMA and with wgs_per_cu = 2.  The plain MFMA loop is also built for    */
                       /* 256, 768 and 1024 threads (the last two leave too few registers and    */
                       /* spill: correct, slower)                                                 */
-  int pipeline;       /* MFMA tile loop: 0 = default: loop 2 at 512 threads, loop 3 otherwise;   */
-                      /* 2 = loads issued two tiles ahead with explicit waits (512 threads only: */
-                      /* asking for it with another size is an error),                           */
+  int pipeline;       /* MFMA tile loop: 0 = default: loop 4 at 512 threads, loop 3 otherwise;   */
+                      /* 4 = loads issued two tiles ahead with explicit waits, hidden units      */
+                      /* 32 .. 39 on v_mfma_f32_4x4x1_16b_f32 blocks (512 threads only: asking   */
+                      /* for it with another size is an error), 2 = the same loop with three     */
+                      /* 16-wide hidden tiles (the last one half empty; 512 threads only),       */
                       /* 1 = software-pipelined GEMM/pointwise stages (512 or 256 threads),      */
                       /* 3 = plain loop (256, 512, 768 or 1024 threads)                          */
   int transitions_per_launch; /* bound on one kernel's run time (default 5; 1 for 64 -> 128 -> 1);       */

@@ -161,11 +161,12 @@ int make_plan_uncached(const bnnhmc_model& m, const bnnhmc_launch* lp, const Dev
     return fail(BNNHMC_ERR_INVALID, "unknown layer variant %d", l.layer);
   if (l.wgs_per_cu < 1 || l.wgs_per_cu > 2)
     return fail(BNNHMC_ERR_INVALID, "wgs_per_cu must be 1 or 2, got %d", l.wgs_per_cu);
-  // MFMA tile loop: 0 / 2 = explicitly prefetched loop (default), 1 = software-pipelined, 3 = plain
+  // MFMA tile loop: 0 / 4 = prefetched loop with hidden units 32 .. 39 on 4x4 blocks (default), 2 = prefetched
+  // loop with three 16-wide hidden tiles, 1 = software-pipelined, 3 = plain
   int loop = 0;
-  if (l.layer == BNNHMC_LAYER_MFMA) loop = l.pipeline == 1 ? 1 : (l.pipeline == 3 ? 0 : (l.pipeline == 4 ? 4 : 2));
-  // the prefetched loop exists for 512 threads only; other sizes get the plain loop unless the
-  // prefetched one was asked for by name (then there is no kernel, reported below)
+  if (l.layer == BNNHMC_LAYER_MFMA) loop = l.pipeline == 1 ? 1 : (l.pipeline == 3 ? 0 : (l.pipeline == 2 ? 2 : 4));
+  // the prefetched loops exist for 512 threads only; other sizes get the plain loop unless a prefetched
+  // one was asked for by name (then there is no kernel, reported below)
   if (l.layer == BNNHMC_LAYER_MFMA && l.pipeline == 0 && l.threads > 0 && l.threads != 512) loop = 0;
   p.wide = m.d0 == 64 && m.d1 == 128;
   if (p.wide) {

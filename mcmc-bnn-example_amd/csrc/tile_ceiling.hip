@@ -16,6 +16,7 @@
 #include <cstdlib>
 #include <vector>
 
+#include "bnn_mfma_hybrid_layer.h"
 #include "bnn_mfma_layer.h"
 #include "bnn_mfma_wide_layer.h"
 
@@ -303,6 +304,52 @@ __global__ __launch_bounds__(512) void hybrid_kernel(float* out, unsigned long l
 }
 
 // ------------------------------------------------------------------------------------------------
+// The tile the kernel runs by default: MfmaHybridLayer::compute_tile (hidden 32 .. 39 on 4x4 blocks in both
+// contractions, the block operands read from the wave's LDS copy of the tile), on a tile held in registers.
+// ------------------------------------------------------------------------------------------------
+using Hybrid = MfmaHybridLayer<22, 40>;
+__global__ __launch_bounds__(512) void hybrid_layer_kernel(float* out, unsigned long long* cycles, int tiles,
+                                                           ModelConsts mc, const float* w) {
+  __shared__ float s_w[Hybrid::P_AL];
+  __shared__ __align__(16) float s_tile[8][Hybrid::TILE_LDS];
+  for (int p = threadIdx.x; p < Hybrid::P; p += blockDim.x) s_w[p] = w[p];
+  __syncthreads();
+  const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+  Hybrid layer;
+  layer.load_weights<1>(s_w, mc);
+  layer.zero_acc();
+  StepCtx cx;
+  cx.n = 1 << 30;
+  cx.ell_prev = nullptr;
+  cx.ell_new = nullptr;
+  Hybrid::TileIn ti;
+  for (int i = 0; i < Hybrid::KP; ++i) ti.xa[i] = f2{0.01f * (lane + i), -0.02f * (lane - i)};
+  for (int j = 0; j < 4; ++j) ti.xe[j] = 0.02f * (n - j);
+  ti.y1 = 0.1f * q;
+  float* tile = s_tile[threadIdx.x >> 6];
+  const unsigned long long c0 = __builtin_readcyclecounter();
+  const unsigned long long r0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < tiles; ++it) {
+    asm volatile("" : "+v"(ti.xa[0]), "+v"(ti.xa[1]), "+v"(ti.xa[2]), "+v"(ti.xe[0]), "+v"(ti.xe[1]),
+                      "+v"(ti.xe[2]), "+v"(ti.xe[3]), "+v"(ti.y1));
+    layer.compute_tile<1, false, true>(ti, tile, cx, mc, 0, n, q);
+  }
+  const unsigned long long c1 = __builtin_readcyclecounter();
+  float sum = layer.dw2s5 + layer.hs;
+  for (int fs = 0; fs < 6; ++fs)
+    for (int j = 0; j < 4; ++j) sum += layer.d5[fs][j];
+  for (int t = 0; t < Hybrid::NT; ++t) {
+    sum += layer.dw2s[t];
+    for (int j = 0; j < 4; ++j) sum += layer.dacc_e[t][j] + layer.dacc_f[t][0][j] + layer.dacc_f[t][1][j];
+  }
+  out[blockIdx.x * blockDim.x + threadIdx.x] = sum;
+  if (threadIdx.x == 0) {
+    cycles[2 * blockIdx.x] = c1 - c0;
+    cycles[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // The tile of the 64 -> 128 -> 1 kernel: MfmaWideLayer::compute_tile on a tile held in registers, the
 // weights in LDS as in the kernel, 256 threads per workgroup = one wave per SIMD.
 // ------------------------------------------------------------------------------------------------
@@ -420,6 +467,7 @@ int main(int argc, char** argv) {
   if (run(tile_kernel<2>, "the pointwise stage alone", tiles, d_out, d_cyc, mc, d_w)) return 1;
   if (run(hybrid_kernel<1>, "hidden 32..39 on 4x4 blocks: GEMM1", tiles, d_out, d_cyc, mc, d_w)) return 1;
   if (run(hybrid_kernel<2>, "hidden 32..39 on 4x4 blocks: both", tiles, d_out, d_cyc, mc, d_w)) return 1;
+  if (run(hybrid_layer_kernel, "the same as the kernel runs it (LDS)", tiles, d_out, d_cyc, mc, d_w)) return 1;
   const int wt = tiles / 5 > 0 ? tiles / 5 : 1;
   std::printf("tile of 16 rows, 64 -> 128 -> 1, one wave per SIMD, %d tiles per wave, 256 workgroups of 256 threads\n", wt);
   if (run(wide_kernel<3>, "whole tile (MFMAs + pointwise)", wt, d_out, d_cyc, mc, d_w, 256)) return 1;

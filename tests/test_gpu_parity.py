@@ -90,13 +90,16 @@ def test_eval_matches_oracle(pkg, lib, orc, layer, kind, n, G):
     s.close()
 
 
-@pytest.mark.parametrize("pipeline,threads", [(1, 512), (3, 512), (3, 768), (3, 1024)])
-def test_alternative_tile_loops_match_oracle(pkg, lib, orc, pipeline, threads):
-    """The software-pipelined (1) and plain (3) tile loops and other workgroup sizes stay selectable
-    through the launch parameters; they must give the same gradients as the default loop."""
-    say("tile loop %d, %d threads" % (pipeline, threads))
+@pytest.mark.parametrize("kind", ["gauss", "t"])
+@pytest.mark.parametrize("pipeline,threads", [(1, 512), (2, 512), (3, 512), (3, 768), (3, 1024), (4, 512)])
+def test_alternative_tile_loops_match_oracle(pkg, lib, orc, pipeline, threads, kind):
+    """The software-pipelined (1), prefetched (2: three 16-wide hidden tiles) and plain (3) tile loops and
+    other workgroup sizes stay selectable through the launch parameters; they must give the same gradients as
+    the default loop (4: hidden units 32 .. 39 on 4x4 blocks), here asked for by name.  4101 rows: 256 full
+    tiles and a ragged one."""
+    say("tile loop %d, %d threads, %s" % (pipeline, threads, kind))
     n = 4101
-    model, om, gen = models(pkg, lib, "gauss", n)
+    model, om, gen = models(pkg, lib, kind, n)
     s = lib.create(model, lib.default_hmc(seed=2), lib.default_launch(cus_per_chain=4, pipeline=pipeline,
                                                                       threads=threads), 1, 1)
     th = s.generate_window(0, **gen)
@@ -112,8 +115,10 @@ def test_alternative_tile_loops_match_oracle(pkg, lib, orc, pipeline, threads):
 def test_prefetched_loop_is_refused_where_it_would_spill(pkg, lib):
     # the loop whose loads come from inline assembly is built for 512 threads only; asking for it by
     # name with another workgroup size is an error, leaving the loop unspecified selects the plain one
-    with pytest.raises(pkg.BnnHmcError):
-        lib.create(lib.default_model(n=64), lib.default_hmc(), lib.default_launch(pipeline=2, threads=1024), 1, 1)
+    for pipeline in (2, 4):
+        with pytest.raises(pkg.BnnHmcError):
+            lib.create(lib.default_model(n=64), lib.default_hmc(),
+                       lib.default_launch(pipeline=pipeline, threads=1024), 1, 1)
     s = lib.create(lib.default_model(n=64), lib.default_hmc(), lib.default_launch(threads=1024), 1, 1)
     s.close()
 
