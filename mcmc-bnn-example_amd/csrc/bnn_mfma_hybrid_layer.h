@@ -183,6 +183,16 @@ struct MfmaHybridLayer {
     }
 #pragma unroll
     for (int s = 0; s < 12; ++s) acc5 = mfma4(x5a[s >> 2][s & 3], w5[s], acc5);
+    // The twelve block instructions accumulate into one register quadruple, each waiting for its predecessor;
+    // the exponentials of the hidden units 0 .. 31 (which only need the wide instructions' results) are
+    // dealt into the gaps: after the wide instructions and the first four block instructions, one
+    // transcendental after every block instruction.
+    float ex[NT][4];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ex[t][j] = __builtin_amdgcn_exp2f(acc[t][j]);
+    }
     // the GEMM2 operands that come from the LDS copy: issued here, used after the pointwise stage
     f2 xf[4];      // x_aug[row 4 q + j][16 + 2 r, 17 + 2 r]
     f2 x5b[2][3];  // x_aug[row ra + rho][6 r .. 6 r + 5]
@@ -194,6 +204,12 @@ struct MfmaHybridLayer {
       x5b[rh][0] = src[0];
       x5b[rh][1] = src[1];
       x5b[rh][2] = src[2];
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);  // 12 wide + 4 block matrix instructions
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);  // one transcendental
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one block matrix instruction
     }
     __builtin_amdgcn_sched_barrier(0);
     // ---- the two k-halves of hidden 32 .. 39: lanes n < 8 keep rows 4 q, 4 q + 1 (registers 0, 1), lanes
@@ -214,8 +230,7 @@ struct MfmaHybridLayer {
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float e = __builtin_amdgcn_exp2f(acc[t][j]);
-        const float sg = __builtin_amdgcn_rcpf(1.0f + e);
+        const float sg = __builtin_amdgcn_rcpf(1.0f + ex[t][j]);
         acc[t][j] = sg;
         yh[j] = __builtin_fmaf(w2g[t], sg, yh[j]);
       }
