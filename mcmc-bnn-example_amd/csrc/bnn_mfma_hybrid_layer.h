@@ -64,7 +64,6 @@ struct MfmaHybridLayer {
 
   struct TileIn {
     f2 xa[KP];   // GEMM1 operand: row n, k = 6 q + 2 i, + 1
-    float xe[4]; // GEMM2 operand: feature n of rows 4 q + j
     float y1;    // target of row 4 q + (n >> 2)
   };
 
@@ -137,8 +136,6 @@ struct MfmaHybridLayer {
       if (k0 >= D0) v = f2{k0 == D0 ? 1.0f : 0.0f, 0.0f};
       ti.xa[i] = v;
     }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) ti.xe[j] = cx.X[(size_t)min(row0 + 4 * q + j, last) * D0 + n];
     ti.y1 = cx.y[min(row0 + 4 * q + (n >> 2), last)];
   }
 
@@ -183,19 +180,12 @@ struct MfmaHybridLayer {
     }
 #pragma unroll
     for (int s = 0; s < 12; ++s) acc5 = mfma4(x5a[s >> 2][s & 3], w5[s], acc5);
-    // The twelve block instructions accumulate into one register quadruple, each waiting for its predecessor;
-    // the exponentials of the hidden units 0 .. 31 (which only need the wide instructions' results) are
-    // dealt into the gaps: after the wide instructions and the first four block instructions, one
-    // transcendental after every block instruction.
-    float ex[NT][4];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) ex[t][j] = __builtin_amdgcn_exp2f(acc[t][j]);
-    }
     // the GEMM2 operands that come from the LDS copy: issued here, used after the pointwise stage
+    float xe[4];   // x[row 4 q + j][n]
     f2 xf[4];      // x_aug[row 4 q + j][16 + 2 r, 17 + 2 r]
     f2 x5b[2][3];  // x_aug[row ra + rho][6 r .. 6 r + 5]
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xe[j] = tile[(4 * q + j) * 24 + n];
 #pragma unroll
     for (int j = 0; j < 4; ++j) xf[j] = *reinterpret_cast<const f2*>(tile + (4 * q + j) * 24 + 16 + 2 * r);
 #pragma unroll
@@ -204,12 +194,6 @@ struct MfmaHybridLayer {
       x5b[rh][0] = src[0];
       x5b[rh][1] = src[1];
       x5b[rh][2] = src[2];
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);  // 12 wide + 4 block matrix instructions
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);  // one transcendental
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one block matrix instruction
     }
     __builtin_amdgcn_sched_barrier(0);
     // ---- the two k-halves of hidden 32 .. 39: lanes n < 8 keep rows 4 q, 4 q + 1 (registers 0, 1), lanes
@@ -230,7 +214,8 @@ struct MfmaHybridLayer {
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float sg = __builtin_amdgcn_rcpf(1.0f + ex[t][j]);
+        const float e = __builtin_amdgcn_exp2f(acc[t][j]);
+        const float sg = __builtin_amdgcn_rcpf(1.0f + e);
         acc[t][j] = sg;
         yh[j] = __builtin_fmaf(w2g[t], sg, yh[j]);
       }
@@ -324,8 +309,8 @@ struct MfmaHybridLayer {
     // ---- GEMM2 ----
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      dacc_e[0] = mfma16(ug[0][j], ti.xe[j], dacc_e[0]);
-      dacc_e[1] = mfma16(ug[1][j], ti.xe[j], dacc_e[1]);
+      dacc_e[0] = mfma16(ug[0][j], xe[j], dacc_e[0]);
+      dacc_e[1] = mfma16(ug[1][j], xe[j], dacc_e[1]);
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -344,7 +329,7 @@ struct MfmaHybridLayer {
 
   // ---- explicitly prefetched loop (see MfmaLayer::prefetch_loop): loads issued from inline assembly two tiles
   //      ahead into three rotating register sets, explicit waits ----
-  static constexpr int N_LOADS = 7;
+  static constexpr int N_LOADS = 3;
   struct TileRaw {
     f4 xa01;   // GEMM1 operand, k-pairs 0 and 1
     TileIn t;  // t.xa[2]: k-pair 2 (the (1, 0) constant in lane group q = 3); t.xa[0 .. 1] from xa01 at use
@@ -352,20 +337,18 @@ struct MfmaHybridLayer {
   template <int N>
   static __device__ __forceinline__ void wait_tile(TileRaw& r) {
     asm volatile("s_waitcnt vmcnt(%[cnt])"
-                 : "+v"(r.xa01), "+v"(r.t.xa[KP - 1]), "+v"(r.t.xe[0]), "+v"(r.t.xe[1]), "+v"(r.t.xe[2]),
-                   "+v"(r.t.xe[3]), "+v"(r.t.y1)
+                 : "+v"(r.xa01), "+v"(r.t.xa[KP - 1]), "+v"(r.t.y1)
                  : [cnt] "n"(N)
                  : "memory");
   }
   struct LoadPlan {
-    unsigned oa, ol, oe, oy;
+    unsigned oa, ol, oy;
     unsigned long long mask_a;
   };
   static __device__ __forceinline__ LoadPlan load_plan(int n, int q) {
     LoadPlan lp;
     lp.oa = (unsigned)((n * D0 + KS * q) * 4);
     lp.ol = lp.oa + 2 * (KP - 1) * 4;
-    lp.oe = (unsigned)(((4 * q) * D0 + n) * 4);
     lp.oy = (unsigned)((4 * q + (n >> 2)) * 4);
     const bool a_const = KS * q + 2 * (KP - 1) >= D0;
     lp.mask_a = __builtin_amdgcn_ballot_w64(!a_const);
@@ -381,18 +364,12 @@ struct MfmaHybridLayer {
         "s_mov_b64 %[sv], exec\n\t"
         "s_nop 3\n\t"
         "global_load_dwordx4 %[xa01], %[oa], %[bx]\n\t"
-        "global_load_dword %[xe0], %[oe], %[bx]\n\t"
-        "global_load_dword %[xe1], %[oe], %[bx] offset:%[r1]\n\t"
-        "global_load_dword %[xe2], %[oe], %[bx] offset:%[r2]\n\t"
-        "global_load_dword %[xe3], %[oe], %[bx] offset:%[r3]\n\t"
         "global_load_dword %[y1], %[oy], %[by]\n\t"
         "s_and_b64 exec, %[sv], %[ma]\n\t"
         "global_load_dwordx2 %[xa2], %[ol], %[bx]\n\t"
         "s_mov_b64 exec, %[sv]"
-        : [xa01] "=&v"(r.xa01), [xa2] "+v"(r.t.xa[KP - 1]), [xe0] "=&v"(r.t.xe[0]), [xe1] "=&v"(r.t.xe[1]),
-          [xe2] "=&v"(r.t.xe[2]), [xe3] "=&v"(r.t.xe[3]), [y1] "=&v"(r.t.y1), [sv] "=&s"(exec_save)
-        : [oa] "v"(lp.oa), [ol] "v"(lp.ol), [oe] "v"(lp.oe), [oy] "v"(lp.oy), [bx] "s"(bx), [by] "s"(by),
-          [ma] "s"(lp.mask_a), [r1] "n"(D0 * 4), [r2] "n"(2 * D0 * 4), [r3] "n"(3 * D0 * 4)
+        : [xa01] "=&v"(r.xa01), [xa2] "+v"(r.t.xa[KP - 1]), [y1] "=&v"(r.t.y1), [sv] "=&s"(exec_save)
+        : [oa] "v"(lp.oa), [ol] "v"(lp.ol), [oy] "v"(lp.oy), [bx] "s"(bx), [by] "s"(by), [ma] "s"(lp.mask_a)
         : "memory", "scc");
   }
 

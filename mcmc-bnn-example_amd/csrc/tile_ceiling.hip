@@ -324,14 +324,12 @@ __global__ __launch_bounds__(512) void hybrid_layer_kernel(float* out, unsigned 
   cx.ell_new = nullptr;
   Hybrid::TileIn ti;
   for (int i = 0; i < Hybrid::KP; ++i) ti.xa[i] = f2{0.01f * (lane + i), -0.02f * (lane - i)};
-  for (int j = 0; j < 4; ++j) ti.xe[j] = 0.02f * (n - j);
   ti.y1 = 0.1f * q;
   float* tile = s_tile[threadIdx.x >> 6];
   const unsigned long long c0 = __builtin_readcyclecounter();
   const unsigned long long r0 = __builtin_amdgcn_s_memrealtime();
   for (int it = 0; it < tiles; ++it) {
-    asm volatile("" : "+v"(ti.xa[0]), "+v"(ti.xa[1]), "+v"(ti.xa[2]), "+v"(ti.xe[0]), "+v"(ti.xe[1]),
-                      "+v"(ti.xe[2]), "+v"(ti.xe[3]), "+v"(ti.y1));
+    asm volatile("" : "+v"(ti.xa[0]), "+v"(ti.xa[1]), "+v"(ti.xa[2]), "+v"(ti.y1));
     layer.compute_tile<1, false, true>(ti, tile, cx, mc, 0, n, q);
   }
   const unsigned long long c1 = __builtin_readcyclecounter();
