@@ -514,6 +514,10 @@ struct MfmaHybridLayer {
   template <int LIK>
   __device__ __forceinline__ void write_partials(float* slot, const float*, bool last) {
     const int lane = opaque_tid() & 63, n = lane & 15, q = lane >> 4, r = n & 3, cb = n >> 2;
+    // The lane swaps below read the accumulators from inside assembly statements, where the compiler does not
+    // count the wait states a vector instruction needs after a matrix instruction wrote its operand (up to 11
+    // for the wide ones).  Once per step: sixteen wait states here cover whatever the tile loop ended on.
+    asm volatile("s_nop 15" ::: "memory");
     // ---- hidden 0 .. 31, features 0 .. 15: lane (n, q), component i: c = 16 t + 4 q + i, f = n ----
 #pragma unroll
     for (int t = 0; t < NT; ++t) *reinterpret_cast<f4*>(slot + n * ROW + 16 * t + 4 * q) = dacc_e[t];
