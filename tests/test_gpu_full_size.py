@@ -545,3 +545,52 @@ def test_reference_model_first_transitions_at_full_size(pkg, lib, orc):
     assert clear.sum() >= n2 - 1
     assert np.all(np.abs(la_gpu - la_ref) <= tol)
     assert 3 <= acc_gpu.sum() <= n2 - 3, "the step size was chosen so that accepts and rejects mix"
+
+
+def test_posterior_moments_over_800_samples_with_all_rows(pkg, lib, orc):
+    """north-star: posterior mean/std of every weight within Monte-Carlo error over 800 samples -- here with all
+    58368 rows in every gradient.  The benchmark configurations themselves cannot decide it (1000-step
+    trajectories cost the oracle 48 minutes, and their chains do not mix within 800 samples: split R-hat above
+    1.1 for 95 % of the weights), so this is a posterior that does mix and that the oracle can afford: Gaussian
+    likelihood sigma = 2, prior N(0, 0.05^2), 25 leapfrog steps, eps0 = 0.005 with the reference's adaptation
+    (accept rate 0.77; two ORACLE chains with different seeds: max z 3.5 over the 961 weights, 0.3 % above 3, std
+    ratios in [0.88, 1.16]).  The GPU's and the oracle's chain share the RNG stream and take the same decisions
+    until rounding parts them, then they are two realisations of one sampler: batch-means standard errors."""
+    import math
+
+    n, L, burn, keep, seed = N_FULL, 25, 100, 800, 33
+    say("posterior moments with all rows: 900 transitions of 25 leapfrog steps")
+    model = lib.default_model(n=n, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=2.0, prior_scale=0.05)
+    om = ob.Model(D0, D1, n, ob.LIK_GAUSSIAN, 2.0, 0.0, 0.05)
+    hmc = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=0.005, seed=seed)
+    s = lib.create(model, hmc, lib.default_launch(transitions_per_launch=50), 1, 1)
+    s.generate_window(0, teacher_scale=0.1, noise_sigma=0.01)
+    X, y = s.get_window_data(0)
+    s.init_chains(None)
+    s.run(burn + keep)
+    a = s.get_samples(0).astype(np.float64)
+    tr = s.get_traces(0)
+    s.close()
+    t0 = time.time()
+    ref = orc.run_chain(om, ob.Hmc(L, burn, keep, burn, 0.005, 0.2, 0.1, 0.01, seed, 0), X, y)
+    b = ref["samples"].astype(np.float64)
+    same = int(np.argmax(tr["accept"] != ref["accept"])) if np.any(tr["accept"] != ref["accept"]) else burn + keep
+    say("oracle chain in %.0f s; accept rate gpu %.3f oracle %.3f; the first %d decisions are the same" % (
+        time.time() - t0, tr["accept"].mean(), ref["accept"].mean(), same))
+    assert a.shape == b.shape == (keep, P)
+    assert np.array_equal(tr["accept"][:50], ref["accept"][:50])
+    assert abs(tr["accept"].mean() - ref["accept"].mean()) < 0.05
+    assert 0.5 < ref["accept"].mean() < 0.95
+
+    def batch_means_se(x, nb=20):
+        bm = x.reshape(nb, -1, x.shape[1]).mean(1)
+        return bm.std(0, ddof=1) / math.sqrt(nb)
+
+    se = np.sqrt(batch_means_se(a) ** 2 + batch_means_se(b) ** 2)   # Monte-Carlo error of a difference
+    z = np.abs(a.mean(0) - b.mean(0)) / se
+    ratio = a.std(0) / b.std(0)
+    say("max z %.2f, fraction above 3: %.4f, std ratios in [%.3f, %.3f]" % (z.max(), np.mean(z > 3.0), ratio.min(),
+                                                                            ratio.max()))
+    assert z.max() < 5.0, "a posterior mean is off by %.2f Monte-Carlo standard errors" % z.max()
+    assert np.mean(z > 3.0) < 0.02
+    assert 0.75 < ratio.min() and ratio.max() < 1.33
