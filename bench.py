@@ -7,8 +7,9 @@ N(0, 0.01^2) noise, Gaussian likelihood, Gaussian weight prior), one chain per w
 leapfrog steps per transition, all 200 windows resident in HBM (1.07 GB).  A "step" is one HMC transition
 (momentum resampling, 1000 fused leapfrog gradient evaluations, log accept ratio, Metropolis decision,
 sample store) of every one of the 200 windows: the chains take turns, five transitions at a time, on
-launches of 128 chains at 2 workgroups per chain; what does not fill such a launch runs as 64 chains at 4,
-32 at 8, ... workgroups per chain, always over all 256 compute units.  The warm-up transitions
+launches of 32 chains at 8 workgroups per chain (the rows of 32 windows, 172 MB, stay in the memory-side
+cache from one leapfrog step to the next); what does not fill such a launch runs as 16 chains at 16, 8 at
+32, ... workgroups per chain, always over all 256 compute units.  The warm-up transitions
 are the burn-in (nothing stored), the timed ones store their samples.  The metric is leapfrog gradient
 evaluations per second; the minutes for 200 windows x (100 burn-in + 800 samples) are 900 steps plus the
 bootstrap evaluation, and --full runs that whole job.
@@ -45,10 +46,11 @@ def measured_traffic(kernel_key):
         return None
 
 
-def batch_plan(n_chains, resident_wgs, cus_per_chain, wide):
+def batch_plan(n_chains, resident_wgs, cus_per_chain, wide, max_chains):
     """[(chains, workgroups per chain)] of the launches that cover n_chains, as the library lays them out:
     a fixed group size when one is configured (the 64->128->1 default is 4), otherwise the largest
-    power-of-two number of chains that is left and fits, spread over the whole device; a batch that
+    power-of-two number of chains that is left and fits (max_chains: what the library says fits, which
+    also keeps a launch's rows inside the memory-side cache), spread over the whole device; a batch that
     leaves compute units idle gets its groups doubled while they still fit."""
     def widen(g, b):
         while g * 2 * b <= resident_wgs and g * 2 <= 256:
@@ -62,7 +64,7 @@ def batch_plan(n_chains, resident_wgs, cus_per_chain, wide):
             g = fixed if cus_per_chain else widen(fixed, b)
         else:
             b = 1
-            while b * 2 <= min(left, resident_wgs):
+            while b * 2 <= min(left, resident_wgs, max_chains):
                 b *= 2
             g = widen(1, b)
         out.append((b, g))
@@ -153,8 +155,6 @@ def main():
     resident_wgs = cus * wgs_per_cu
     n_windows = args.windows or (max(1, resident_wgs // 4 // cpw) if wide else 200)
     n_chains = n_windows * cpw
-    plan = batch_plan(n_chains, resident_wgs, launch.cus_per_chain, wide)
-    resident = plan[0][0]                                   # chains in flight in the first launches
 
     student = args.lik == "student_t"
     if student:
@@ -172,6 +172,9 @@ def main():
     if not args.full:
         hmc.eps0 = args.eps0
     s = lib.create(model, hmc, launch, n_windows, cpw)
+    plan = batch_plan(n_chains, resident_wgs, launch.cus_per_chain, wide, s.batching()[0])
+    resident = plan[0][0]                                   # chains in flight in the first launches
+    assert plan[0] == s.batching(), (plan[0], s.batching())
     teachers = []
     t_gen = time.perf_counter()
     for w in range(n_windows):
@@ -254,7 +257,7 @@ def main():
                 "%d x %d, the %d chains taking turns in quanta of %d transitions; what does not fill a launch runs "
                 "in the largest batches that fit (%s)" % (
                     plan[0][0], plan[0][1], n_chains, args.transitions_per_launch,
-                    ", ".join("%d x %d" % bg for bg in plan[1:]))
+                    ", ".join("%d x %d" % bg for bg in sorted(set(plan[1:]), reverse=True)))
                 if not wide and not launch.cus_per_chain and len(plan) > 1
                 else ", ".join("%d x %d" % bg for bg in plan)),
             "workgroups_last_launch": tm1["workgroups"], "compute_units": cus,

@@ -73,8 +73,10 @@ typedef struct bnnhmc_launch {
   int layer;          /* BNNHMC_LAYER_MFMA (v_mfma_f32_16x16x4_f32, _4x4x1_16b_f32) or BNNHMC_LAYER_FFMA */
   int cus_per_chain;  /* workgroups that share one chain's rows; 0 = automatic.  Sampler,         */
                       /* 22 -> 40 -> 1: a batch is the largest power-of-two number of chains that */
-                      /* fits, spread over the whole device (one chain: 256 workgroups; 128 or     */
-                      /* more chains on 256 CUs: 2 each); more chains than fit take turns on such  */
+                      /* fits and whose windows' rows stay within 192 MB (the memory-side cache),  */
+                      /* spread over the whole device (one chain: 256 workgroups; 32 or more       */
+                      /* windows of 58368 x 22 on 256 CUs: 8 each; small windows: down to 2 each;  */
+                      /* see bnnhmc_get_batching); more chains than fit take turns on such         */
                       /* batches, transitions_per_launch transitions at a time, and what does not  */
                       /* fill a batch runs in smaller, wider ones.  64 -> 128 -> 1: 4, a smaller    */
                       /* last batch widened.  Step operator: 256.  Results are bit-reproducible for */
@@ -263,6 +265,14 @@ int bnnhmc_eval(bnnhmc_sampler* s, int window, const float* w, float* ell, float
 /* Mean over one chain's kept samples of the data log-likelihood, the log-prior and their sum
  * (output_final_loss, main.h:78-115). */
 int bnnhmc_final_loss(bnnhmc_sampler* s, int chain, double* loss1, double* loss2, double* full);
+
+/* How bnnhmc_run lays the sampler's chains over the device: chains in a full launch and workgroups per
+ * chain in it.  With the automatic group size (cus_per_chain = 0) of the 22 -> 40 -> 1 kernel a launch takes
+ * the largest power-of-two number of chains that (a) fits the device at one workgroup per chain and (b)
+ * keeps the rows of its windows within 192 MB, so that after the first leapfrog step they are served by the
+ * memory-side cache instead of HBM: 200 windows of 58368 x 22 run 32 at a time on 8 workgroups each.  No
+ * counterpart in the reference (one chain per process). */
+int bnnhmc_get_batching(bnnhmc_sampler* s, int* chains_per_launch, int* workgroups_per_chain);
 
 /* Timing of the work done by bnnhmc_run so far: milliseconds between HIP events recorded on the
  * sampler's stream around the trajectory kernels, number of those launches, gradient evaluations

@@ -56,6 +56,7 @@ EXPORTS = [
     "bnnhmc_get_chain_state", "bnnhmc_get_traces", "bnnhmc_eval", "bnnhmc_final_loss",
     "bnnhmc_get_timing", "bnnhmc_read_reference_data", "bnnhmc_set_chain_state",
     "bnnhmc_split_rhat_ess", "bnnhmc_window_diagnostics", "bnnhmc_step_launch_info",
+    "bnnhmc_get_batching",
 ]
 
 
@@ -317,6 +318,12 @@ class Sampler:
         self.lib.check(self.lib.c.bnnhmc_window_diagnostics(
             self.h, window, rhat.ctypes.data_as(C.c_void_p), ess.ctypes.data_as(C.c_void_p)))
         return rhat, ess
+
+    def batching(self):
+        """(chains in a full launch, workgroups per chain in it)"""
+        b, g = C.c_int(), C.c_int()
+        self.lib.check(self.lib.c.bnnhmc_get_batching(self.h, C.byref(b), C.byref(g)))
+        return b.value, g.value
 
     def timing(self):
         ms, launches, evals, wgs = C.c_double(), C.c_long(), C.c_long(), C.c_int()

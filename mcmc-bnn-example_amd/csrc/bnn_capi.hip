@@ -129,6 +129,27 @@ int env_pipeline() {
   const char* e = getenv("BNNHMC_PIPELINE");
   return e && *e ? atoi(e) : 0;
 }
+// The rows of the windows of a launch are read again at every leapfrog step.  A batch whose windows fit the
+// 256 MB memory-side cache gets them from there after the first step; a wider one streams them from HBM
+// (2.3 TB/s at 128 windows of 58368 x 22 on 2 workgroups each).  What that costs depends on the card --
+// evaluations/s of 128 windows at 2 workgroups per chain / 64 at 4 / 32 at 8, each batch filling the device:
+// 419 k / 415 k / 415 k on one MI355X, 395 k / 396 k / 415 k on another -- so with the automatic group size a
+// batch takes no more windows than fit this budget (32 of that size: 172 MB).
+// BNNHMC_RESIDENT_MB=<n> replaces it for measurements (0: no limit).
+size_t resident_row_budget() {
+  const char* e = getenv("BNNHMC_RESIDENT_MB");
+  const long mb = e && *e ? atol(e) : 192;
+  return mb <= 0 ? (size_t)0 : (size_t)mb << 20;
+}
+// chains of a batch whose windows' rows fit the budget (0: no limit)
+int resident_chain_cap(const bnnhmc_model& m, int chains_per_window) {
+  const size_t budget = resident_row_budget();
+  const size_t window_bytes = (size_t)m.n * (size_t)(m.d0 + 1) * sizeof(float);
+  if (budget == 0 || window_bytes > budget) return 0;  // nothing fits anyway: fewest exchanges win
+  const size_t windows = budget / window_bytes;
+  return (int)std::min<size_t>(windows * (size_t)chains_per_window, (size_t)1 << 20);
+}
+
 // How a launch is laid over the GPU
 struct Plan {
   const void* kernel = nullptr;
@@ -196,9 +217,9 @@ int make_plan_uncached(const bnnhmc_model& m, const bnnhmc_launch* lp, const Dev
   const int resident = p.wgs_per_cu * di.cus;
   p.resident_wgs = resident;
   // 0 = automatic.  22 -> 40 -> 1: a batch is the largest power-of-two number of chains that is left
-  // and fits (one workgroup per chain at least), each chain on resident / batch workgroups -- 200
-  // chains on 256 CUs run as 128 x 2, 64 x 4, 8 x 32 (measured, evaluations/s with every CU busy:
-  // 2 workgroups per chain 386 k, 4: 379 k, 8: 368 k, 16: 341 k, 32: 289 k).  64 -> 128 -> 1: 4
+  // and fits (one workgroup per chain at least; a sampler also keeps the rows of a batch within
+  // resident_row_budget()), each chain on resident / batch workgroups (measured, evaluations/s with every
+  // CU busy: 2 workgroups per chain 419 k, 4: 415 k, 8: 415 k, 16: 382 k, 32: 328 k).  64 -> 128 -> 1: 4
   // workgroups per chain, a last smaller batch widened.
   p.G = l.cus_per_chain > 0 ? l.cus_per_chain : (p.wide ? std::min(4, resident) : 1);
   p.widen = l.cus_per_chain <= 0;
@@ -1032,6 +1053,10 @@ int bnnhmc_create(const bnnhmc_model* model, const bnnhmc_hmc* hmc, const bnnhmc
     delete s;
     return rc;
   }
+  if (s->plan.widen && !s->plan.wide) {
+    const int cap = resident_chain_cap(*model, chains_per_window);
+    if (cap > 0 && cap < s->plan.max_groups) s->plan.max_groups = cap;
+  }
   auto bail = [&](int code) {
     bnnhmc_destroy(s);
     return code;
@@ -1507,6 +1532,16 @@ int bnnhmc_window_diagnostics(bnnhmc_sampler* s, int window, double* rhat, doubl
                          host.size() * sizeof(float), hipMemcpyDeviceToHost, s->stream));
   HIP_TRY(hipStreamSynchronize(s->stream));
   return bnnhmc_split_rhat_ess(host.data(), s->cpw, stored, s->L.P, stride, rhat, ess);
+}
+
+int bnnhmc_get_batching(bnnhmc_sampler* s, int* chains_per_launch, int* workgroups_per_chain) {
+  if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
+  const int groups = batch_size(s->plan, s->n_chains);
+  if (chains_per_launch) *chains_per_launch = groups;
+  if (workgroups_per_chain)
+    *workgroups_per_chain =
+        s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs, 256) : s->plan.G;
+  return BNNHMC_OK;
 }
 
 int bnnhmc_get_timing(bnnhmc_sampler* s, double* kernel_ms, long* launches, long* grad_evals,

@@ -250,3 +250,51 @@ def test_step_operator_failure_record_survives_later_steps(pkg, lib, orc, monkey
     lib.step_check(model, launch, ws.ptr, 0)
     ref = orc.mcmc_step(om, X, y, th, m0, g0, np.float32(0.01), L)
     assert float(np.abs(outs[2].numpy(P) - ref[2]).max()) <= 1e-5 * float(np.abs(ref[2]).max())
+
+
+# ------------------------------------------------------------------------------------------------
+# automatic batches keep the rows of their windows inside the memory-side cache
+# ------------------------------------------------------------------------------------------------
+def test_automatic_batches_are_cut_to_the_memory_side_cache(pkg, lib, orc, monkeypatch):
+    """With the automatic group size a launch takes no more windows than 192 MB of rows: 32 windows of
+    58368 x 22 (172 MB) on 8 workgroups each where 64 would fit the device on 4; chains that share a window
+    share its rows (32 windows x 2 chains: 64 on 4); small windows are not cut.  The cut only changes how
+    the chains are laid over the device: the same transitions with the limit lifted (the measurement switch
+    BNNHMC_RESIDENT_MB=0) take the same decisions and differ by the rounding of a different group size."""
+    n_full = 58368
+    hmc = lib.default_hmc(leapfrog_steps=3, burn_in=0, n_samples=2, eps0=2e-5, seed=9)
+    model = lib.default_model(n=n_full, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
+
+    def run(n_windows, cpw, m=model):
+        s = lib.create(m, hmc, lib.default_launch(), n_windows, cpw)
+        b = s.batching()
+        for w in range(n_windows):
+            s.generate_window(w, teacher_scale=0.1, noise_sigma=0.01)
+        s.init_chains(None)
+        s.run(2)
+        out = [s.get_samples(c) for c in (0, n_windows * cpw - 1)], [s.get_traces(c) for c in (0, n_windows * cpw - 1)]
+        s.close()
+        return b, out
+
+    say("64 windows of 58368 rows, automatic group size")
+    b_cut, (smp_cut, tr_cut) = run(64, 1)
+    assert b_cut == (32, 8), b_cut
+    monkeypatch.setenv("BNNHMC_RESIDENT_MB", "0")
+    b_all, (smp_all, tr_all) = run(64, 1)
+    assert b_all == (64, 4), b_all
+    monkeypatch.delenv("BNNHMC_RESIDENT_MB")
+    for a, b, ta, tb in zip(smp_cut, smp_all, tr_cut, tr_all):
+        assert np.array_equal(ta["accept"], tb["accept"])
+        assert np.allclose(ta["log_acpt"], tb["log_acpt"], rtol=2e-3, atol=1e-2), (ta["log_acpt"], tb["log_acpt"])
+        assert np.max(np.abs(a - b)) <= 1e-5 * np.max(np.abs(b))
+    say("32 windows x 2 chains")
+    s = lib.create(model, hmc, lib.default_launch(), 32, 2)
+    assert s.batching() == (64, 4), s.batching()
+    s.close()
+    small = lib.default_model(n=4096, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
+    s = lib.create(small, hmc, lib.default_launch(), 200, 1)
+    assert s.batching() == (128, 2), s.batching()
+    s.close()
+    s = lib.create(model, hmc, lib.default_launch(cus_per_chain=2), 200, 1)   # a configured group size is kept
+    assert s.batching() == (128, 2), s.batching()
+    s.close()

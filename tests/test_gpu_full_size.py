@@ -359,8 +359,8 @@ def test_1600_samples_at_reduced_size(pkg, lib, orc):
 
 
 # ------------------------------------------------------------------------------------------------
-# configs[2] batching: 200 windows of 58368 rows as a batch of 128 (2 workgroups per chain), one of 64
-# (4 per chain) and a last batch of 8 (widened to 32 workgroups per chain)
+# configs[2] batching: 200 windows of 58368 rows as six batches of 32 (8 workgroups per chain: the rows of a
+# batch stay in the memory-side cache) and a last batch of 8 (widened to 32 workgroups per chain)
 # ------------------------------------------------------------------------------------------------
 def test_200_windows_are_batched_without_crosstalk(pkg, lib, orc):
     # a step size small enough that trajectories from the all-zero start are accepted
@@ -372,21 +372,23 @@ def test_200_windows_are_batched_without_crosstalk(pkg, lib, orc):
     for w in range(200):
         big.generate_window(w, teacher_scale=0.1, noise_sigma=0.01)
     big.init_chains(None)
+    big_batching = big.batching()
     say("200 windows: two transitions of every window")
     big.run(burn + keep)
     assert big.timing()["grad_evals"] == 200 * 2 * L
     checks = {}
-    for chain in (0, 63, 64, 127, 128, 150, 191, 192, 199):
+    for chain in (0, 31, 32, 63, 64, 150, 191, 192, 199):
         checks[chain] = (big.get_samples(chain), big.get_traces(chain), big.get_chain_state(chain),
                          big.get_window_data(chain) if chain in (0, 150, 199) else None)
         assert np.all(np.isfinite(checks[chain][0])) and checks[chain][2]["transitions_done"] == 2
         assert checks[chain][2]["n_accepted"] >= 1 and np.abs(checks[chain][0]).max() > 0
     big.close()
-    assert not np.array_equal(checks[63][0], checks[64][0])       # different windows, different chains
-    # chain 0 sat in the batch of 128 at 2 workgroups per chain, chain 150 in the batch of 64 at 4, chain
-    # 199 in the tail batch of 8 at 32: each must equal, bit for bit, a sampler that holds only that
-    # window and is launched that way
-    for chain, G in ((0, 2), (150, 4), (199, 32)):
+    assert not np.array_equal(checks[31][0], checks[32][0])       # different windows, different chains
+    # the rows of 32 such windows fit the memory-side cache, so the 200 chains ran in six batches of 32 at 8
+    # workgroups per chain and a tail batch of 8 at 32: each chain must equal, bit for bit, a sampler that
+    # holds only that window and is launched that way
+    assert big_batching == (32, 8), big_batching
+    for chain, G in ((0, 8), (150, 8), (199, 32)):
         X, y = checks[chain][3]
         h1 = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=eps0, seed=0,
                              adapt_steps=0, chain_id_base=chain)
