@@ -172,9 +172,6 @@ def main():
     if not args.full:
         hmc.eps0 = args.eps0
     s = lib.create(model, hmc, launch, n_windows, cpw)
-    plan = batch_plan(n_chains, resident_wgs, launch.cus_per_chain, wide, s.batching()[0])
-    resident = plan[0][0]                                   # chains in flight in the first launches
-    assert plan[0] == s.batching(), (plan[0], s.batching())
     teachers = []
     t_gen = time.perf_counter()
     for w in range(n_windows):
@@ -211,6 +208,11 @@ def main():
         s.run(steps)  # synchronous at return: the stream is drained
         wall = time.perf_counter() - t0
     tm1 = s.timing()
+    # the batch the library ended up with (where two shapes compete it has timed a launch of each)
+    batching, trial = s.batching(), s.batch_trial_rates()
+    plan = batch_plan(n_chains, resident_wgs, launch.cus_per_chain, wide, batching[0])
+    assert plan[0] == batching, (plan[0], batching)
+    resident = plan[0][0]                                   # chains in flight in a full launch
     states = [s.get_chain_state(c) for c in range(n_chains)]
     stored = s.get_samples(0).shape[0]
     s.close()
@@ -260,6 +262,10 @@ def main():
                     ", ".join("%d x %d" % bg for bg in sorted(set(plan[1:]), reverse=True)))
                 if not wide and not launch.cus_per_chain and len(plan) > 1
                 else ", ".join("%d x %d" % bg for bg in plan)),
+            "batch_shape_trial": None if trial[0] <= 0 else (
+                "the library timed one launch of each shape at the start of the %s: rows of a launch within the "
+                "memory-side cache %.0f evals/s, as many chains as fit the device %.0f evals/s" % (
+                    "job" if args.full else "warm-up call", trial[0], trial[1])),
             "workgroups_last_launch": tm1["workgroups"], "compute_units": cus,
             "transitions_per_launch": args.transitions_per_launch,
             "eps0": float(hmc.eps0), "adapt_steps": int(hmc.adapt_steps),

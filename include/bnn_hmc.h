@@ -73,16 +73,18 @@ typedef struct bnnhmc_launch {
   int layer;          /* BNNHMC_LAYER_MFMA (v_mfma_f32_16x16x4_f32, _4x4x1_16b_f32) or BNNHMC_LAYER_FFMA */
   int cus_per_chain;  /* workgroups that share one chain's rows; 0 = automatic.  Sampler,         */
                       /* 22 -> 40 -> 1: a batch is the largest power-of-two number of chains that */
-                      /* fits and whose windows' rows stay within 192 MB (the memory-side cache),  */
-                      /* spread over the whole device (one chain: 256 workgroups; 32 or more       */
-                      /* windows of 58368 x 22 on 256 CUs: 8 each; small windows: down to 2 each;  */
-                      /* see bnnhmc_get_batching); more chains than fit take turns on such         */
+                      /* fits, spread over the whole device (one chain: 256 workgroups; 128 or     */
+                      /* more chains on 256 CUs: 2 each) -- or, where that is measured to be       */
+                      /* faster, the largest whose windows' rows stay within 192 MB, the           */
+                      /* memory-side cache (32 windows of 58368 x 22: 8 each; see                  */
+                      /* bnnhmc_get_batching); more chains than fit take turns on such             */
                       /* batches, transitions_per_launch transitions at a time, and what does not  */
                       /* fill a batch runs in smaller, wider ones.  64 -> 128 -> 1: 4, a smaller    */
                       /* last batch widened.  Step operator: 256.  Results are bit-reproducible for */
                       /* a fixed count; with 0 and more chains than fit at once, which launches run */
-                      /* wider depends on how a job is cut into bnnhmc_run calls, so a run that     */
-                      /* must be repeatable or resumable bit for bit sets an explicit count         */
+                      /* wider depends on how a job is cut into bnnhmc_run calls and on that time   */
+                      /* measurement, so a run that must be repeatable or resumable bit for bit     */
+                      /* sets an explicit count                                                     */
   int wgs_per_cu;     /* co-resident workgroups per CU, 1 or 2 (default 1)                       */
   int threads;        /* threads per workgroup; default 512 for MFMA (every tile loop), 256 for  */
                       /* FFMA and with wgs_per_cu = 2.  The plain MFMA loop is also built for    */
@@ -266,13 +268,21 @@ int bnnhmc_eval(bnnhmc_sampler* s, int window, const float* w, float* ell, float
  * (output_final_loss, main.h:78-115). */
 int bnnhmc_final_loss(bnnhmc_sampler* s, int chain, double* loss1, double* loss2, double* full);
 
-/* How bnnhmc_run lays the sampler's chains over the device: chains in a full launch and workgroups per
- * chain in it.  With the automatic group size (cus_per_chain = 0) of the 22 -> 40 -> 1 kernel a launch takes
- * the largest power-of-two number of chains that (a) fits the device at one workgroup per chain and (b)
- * keeps the rows of its windows within 192 MB, so that after the first leapfrog step they are served by the
- * memory-side cache instead of HBM: 200 windows of 58368 x 22 run 32 at a time on 8 workgroups each.  No
- * counterpart in the reference (one chain per process). */
-int bnnhmc_get_batching(bnnhmc_sampler* s, int* chains_per_launch, int* workgroups_per_chain);
+/* How bnnhmc_run lays the sampler's chains over the device at present: chains in a full launch and
+ * workgroups per chain in it.  With the automatic group size (cus_per_chain = 0) of the 22 -> 40 -> 1 kernel
+ * a launch takes the largest power-of-two number of chains that fits the device at one workgroup per chain;
+ * where the rows of so many windows exceed 192 MB there is a second shape, the largest such number whose
+ * windows' rows stay within 192 MB, so that after the first leapfrog step they are served by the
+ * memory-side cache instead of HBM (200 windows of 58368 x 22: 32 at a time on 8 workgroups each, against
+ * 128 on 2).  Which is faster depends on the card and on the data (the card is power-limited: HBM traffic
+ * costs shader clock when the arithmetic is dense).  A sampler starts with the cache-resident shape; a
+ * bnnhmc_run call that is long enough (a launch of each shape fits in it) first runs one launch of each,
+ * timed, and goes on with the faster, and so do later calls, which time the two again after every 2000
+ * launches' worth of chains.  trial_rates (may be NULL) receives the gradient evaluations per second of the
+ * last such pair, cache-resident shape first; zeros if none was run.  No counterpart in the reference (one
+ * chain per process). */
+int bnnhmc_get_batching(bnnhmc_sampler* s, int* chains_per_launch, int* workgroups_per_chain,
+                        double* trial_rates);
 
 /* Timing of the work done by bnnhmc_run so far: milliseconds between HIP events recorded on the
  * sampler's stream around the trajectory kernels, number of those launches, gradient evaluations

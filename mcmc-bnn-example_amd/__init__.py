@@ -322,8 +322,14 @@ class Sampler:
     def batching(self):
         """(chains in a full launch, workgroups per chain in it)"""
         b, g = C.c_int(), C.c_int()
-        self.lib.check(self.lib.c.bnnhmc_get_batching(self.h, C.byref(b), C.byref(g)))
+        self.lib.check(self.lib.c.bnnhmc_get_batching(self.h, C.byref(b), C.byref(g), None))
         return b.value, g.value
+
+    def batch_trial_rates(self):
+        """gradient evaluations/s of the last timed pair of launches: (cache-resident shape, device-wide shape)"""
+        r = (C.c_double * 2)()
+        self.lib.check(self.lib.c.bnnhmc_get_batching(self.h, None, None, r))
+        return r[0], r[1]
 
     def timing(self):
         ms, launches, evals, wgs = C.c_double(), C.c_long(), C.c_long(), C.c_int()

@@ -133,9 +133,15 @@ int env_pipeline() {
 // 256 MB memory-side cache gets them from there after the first step; a wider one streams them from HBM
 // (2.3 TB/s at 128 windows of 58368 x 22 on 2 workgroups each).  What that costs depends on the card --
 // evaluations/s of 128 windows at 2 workgroups per chain / 64 at 4 / 32 at 8, each batch filling the device:
-// 419 k / 415 k / 415 k on one MI355X, 395 k / 396 k / 415 k on another -- so with the automatic group size a
-// batch takes no more windows than fit this budget (32 of that size: 172 MB).
-// BNNHMC_RESIDENT_MB=<n> replaces it for measurements (0: no limit).
+// 419 k / 415 k / 415 k on one MI355X, 395 k / 396 k / 415 k on another, and with the reference's Student-t
+// model, whose saturated hidden units put zeros into the second contraction, 427 k / - / 406 k.  The card is
+// power-limited: with the dense Gaussian workload the HBM traffic of the wide batch lowers the shader clock from
+// 2.36 to 2.23 GHz, with the lighter one it does not and the narrow groups' smaller share of exchange time wins.
+// So with the automatic group size a sampler whose chains take turns has two batch shapes -- the largest that
+// fits the device, and the largest whose windows fit this budget (32 of that size: 172 MB) -- and bnnhmc_run
+// times one launch of each at the start of a call and goes on with the faster (tune_batch below).
+// BNNHMC_RESIDENT_MB=<n> replaces the budget for measurements (0: no limit, one shape);
+// BNNHMC_BATCH_TUNE=0 switches the timing off (the cache-resident shape is then used throughout).
 size_t resident_row_budget() {
   const char* e = getenv("BNNHMC_RESIDENT_MB");
   const long mb = e && *e ? atol(e) : 192;
@@ -148,6 +154,11 @@ int resident_chain_cap(const bnnhmc_model& m, int chains_per_window) {
   if (budget == 0 || window_bytes > budget) return 0;  // nothing fits anyway: fewest exchanges win
   const size_t windows = budget / window_bytes;
   return (int)std::min<size_t>(windows * (size_t)chains_per_window, (size_t)1 << 20);
+}
+
+bool env_batch_tune() {
+  const char* e = getenv("BNNHMC_BATCH_TUNE");
+  return !(e && *e && atoi(e) == 0);
 }
 
 // How a launch is laid over the GPU
@@ -378,8 +389,9 @@ int read_status(void* workspace, hipStream_t stream) {
 // Chains of the next batch when `left` are still to run: as many as fit; with the automatic group size
 // of the 22 -> 40 -> 1 kernel the largest power of two of them, so that the batch fills the device with
 // equal groups (see make_plan_uncached).
-int batch_size(const Plan& p, int left) {
+int batch_size(const Plan& p, int left, int limit = 0) {
   int groups = std::min(p.max_groups, left);
+  if (limit > 0) groups = std::min(groups, limit);
   if (p.widen && !p.wide) {
     int b = 1;
     while (b * 2 <= groups) b *= 2;
@@ -550,6 +562,11 @@ struct bnnhmc_sampler {
   std::vector<char> window_set;
   hipStream_t stream = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  hipEvent_t ev_t0 = nullptr, ev_t1 = nullptr;  // around one launch while the batch shape is being chosen
+  int batch_cap = 0;        // chains of a batch whose windows' rows fit the memory-side cache (0: no such limit)
+  int batch_limit = 0;      // the limit bnnhmc_run applies at present: batch_cap or 0 (what fits the device)
+  double tuned_rate[2] = {0.0, 0.0};  // evaluations per ms of the last trial launches: cache-resident, device-wide
+  long quanta_since_tune = -1;        // quanta dealt since the shapes were last timed (-1: never)
   // device memory
   float* X = nullptr;
   float* y = nullptr;
@@ -1055,7 +1072,7 @@ int bnnhmc_create(const bnnhmc_model* model, const bnnhmc_hmc* hmc, const bnnhmc
   }
   if (s->plan.widen && !s->plan.wide) {
     const int cap = resident_chain_cap(*model, chains_per_window);
-    if (cap > 0 && cap < s->plan.max_groups) s->plan.max_groups = cap;
+    if (cap > 0 && cap < s->plan.max_groups) s->batch_cap = s->batch_limit = cap;
   }
   auto bail = [&](int code) {
     bnnhmc_destroy(s);
@@ -1064,6 +1081,8 @@ int bnnhmc_create(const bnnhmc_model* model, const bnnhmc_hmc* hmc, const bnnhmc
   hipError_t e = hipStreamCreate(&s->stream);
   if (e == hipSuccess) e = hipEventCreate(&s->ev0);
   if (e == hipSuccess) e = hipEventCreate(&s->ev1);
+  if (e == hipSuccess) e = hipEventCreate(&s->ev_t0);
+  if (e == hipSuccess) e = hipEventCreate(&s->ev_t1);
   if (e != hipSuccess) {
     fail(BNNHMC_ERR_HIP, "stream/event creation failed: %s", hipGetErrorString(e));
     return bail(BNNHMC_ERR_HIP);
@@ -1107,6 +1126,8 @@ int bnnhmc_destroy(bnnhmc_sampler* s) {
   for (void* p : s->allocs) (void)hipFree(p);
   if (s->ev0) (void)hipEventDestroy(s->ev0);
   if (s->ev1) (void)hipEventDestroy(s->ev1);
+  if (s->ev_t0) (void)hipEventDestroy(s->ev_t0);
+  if (s->ev_t1) (void)hipEventDestroy(s->ev_t1);
   if (s->stream) (void)hipStreamDestroy(s->stream);
   delete s;
   return BNNHMC_OK;
@@ -1171,7 +1192,7 @@ int bnnhmc_init_chains(bnnhmc_sampler* s, const float* w0) {
   // (in the batches the transitions run in when all chains fit at once: a chain's sums are then added
   // in one order for its whole life)
   for (int base = 0, groups = 0; base < s->n_chains; base += groups) {
-    groups = batch_size(s->plan, s->n_chains - base);
+    groups = batch_size(s->plan, s->n_chains - base, s->batch_limit);
     KArgs a = base_args(s);
     a.mode = MODE_STEPS;
     a.L = 1;
@@ -1241,14 +1262,14 @@ int bnnhmc_run(bnnhmc_sampler* s, int n_transitions) {
   // largest batches that fit
   auto run_range = [&](int base, int count, int n_trans) -> int {
     for (int groups = 0; count > 0; count -= groups, base = (base + groups) % s->n_chains) {
-      groups = batch_size(s->plan, count);
+      groups = batch_size(s->plan, count, s->batch_limit);
       const int rc = launch(base, groups, n_trans);
       if (rc) return rc;
     }
     return BNNHMC_OK;
   };
   const int tpl = s->plan.transitions_per_launch;
-  const int full_batch = batch_size(s->plan, s->n_chains);
+  int full_batch = batch_size(s->plan, s->n_chains, s->batch_limit);
   int rc0 = BNNHMC_OK;
   if (s->plan.widen && !s->plan.wide && s->n_chains > full_batch) {
     // More chains than fit at once: they take turns.  A chain's run is cut into quanta of tpl transitions;
@@ -1260,6 +1281,37 @@ int bnnhmc_run(bnnhmc_sampler* s, int n_transitions) {
     // transitions every chain still owes -- runs in the largest batches that fit.
     const long quanta = (long)s->n_chains * (n_transitions / tpl);
     long dealt = 0;
+    // Which of the two batch shapes is faster depends on the card and on the data (see
+    // resident_row_budget): the first launches of a call that is long enough are one of each, timed, and the
+    // call (and the sampler, until a later call measures again) goes on with the faster.  Both do their
+    // share of the work; from here on the results depend on a time measurement -- a run that must be
+    // repeatable bit for bit sets cus_per_chain.
+    const int wide_batch = batch_size(s->plan, s->n_chains);
+    const int narrow_batch = s->batch_cap > 0 ? batch_size(s->plan, s->n_chains, s->batch_cap) : wide_batch;
+    // (again only after kRetuneQuanta more quanta: a trial of the slower shape costs a few per cent of one
+    // launch, and what is faster changes slowly, as the chains burn in)
+    const long kRetuneQuanta = 2000;
+    const bool due = s->quanta_since_tune < 0 || s->quanta_since_tune >= kRetuneQuanta;
+    if (narrow_batch < wide_batch && env_batch_tune() && due && quanta >= narrow_batch + wide_batch) {
+      const int trial[2] = {narrow_batch, wide_batch};
+      for (int k = 0; k < 2 && rc0 == BNNHMC_OK; ++k) {
+        HIP_TRY(hipEventRecord(s->ev_t0, s->stream));
+        rc0 = launch((int)(dealt % s->n_chains), trial[k], tpl);
+        HIP_TRY(hipEventRecord(s->ev_t1, s->stream));
+        HIP_TRY(hipEventSynchronize(s->ev_t1));
+        float tms = 0.0f;
+        HIP_TRY(hipEventElapsedTime(&tms, s->ev_t0, s->ev_t1));
+        s->tuned_rate[k] = tms > 0.0f ? (double)trial[k] * tpl * s->hmc.leapfrog_steps / tms : 0.0;
+        dealt += trial[k];
+      }
+      if (rc0 == BNNHMC_OK) {
+        s->batch_limit = s->tuned_rate[1] > s->tuned_rate[0] ? 0 : s->batch_cap;
+        full_batch = batch_size(s->plan, s->n_chains, s->batch_limit);
+        s->quanta_since_tune = quanta - dealt;
+      }
+    } else if (s->quanta_since_tune >= 0) {
+      s->quanta_since_tune += quanta;
+    }
     for (; rc0 == BNNHMC_OK && quanta - dealt >= full_batch; dealt += full_batch)
       rc0 = launch((int)(dealt % s->n_chains), full_batch, tpl);
     if (rc0 == BNNHMC_OK && quanta > dealt)
@@ -1267,7 +1319,7 @@ int bnnhmc_run(bnnhmc_sampler* s, int n_transitions) {
     if (rc0 == BNNHMC_OK && n_transitions % tpl) rc0 = run_range(0, s->n_chains, n_transitions % tpl);
   } else {
     for (int base = 0, groups = 0; rc0 == BNNHMC_OK && base < s->n_chains; base += groups) {
-      groups = batch_size(s->plan, s->n_chains - base);
+      groups = batch_size(s->plan, s->n_chains - base, s->batch_limit);
       for (int done = 0; rc0 == BNNHMC_OK && done < n_transitions; done += tpl)
         rc0 = launch(base, groups, std::min(tpl, n_transitions - done));
     }
@@ -1534,13 +1586,18 @@ int bnnhmc_window_diagnostics(bnnhmc_sampler* s, int window, double* rhat, doubl
   return bnnhmc_split_rhat_ess(host.data(), s->cpw, stored, s->L.P, stride, rhat, ess);
 }
 
-int bnnhmc_get_batching(bnnhmc_sampler* s, int* chains_per_launch, int* workgroups_per_chain) {
+int bnnhmc_get_batching(bnnhmc_sampler* s, int* chains_per_launch, int* workgroups_per_chain,
+                        double* trial_rates) {
   if (!s) return fail(BNNHMC_ERR_INVALID, "sampler is null");
-  const int groups = batch_size(s->plan, s->n_chains);
+  const int groups = batch_size(s->plan, s->n_chains, s->batch_limit);
   if (chains_per_launch) *chains_per_launch = groups;
   if (workgroups_per_chain)
     *workgroups_per_chain =
         s->plan.widen ? widen_group(s->plan.G, groups, s->plan.resident_wgs, 256) : s->plan.G;
+  if (trial_rates) {
+    trial_rates[0] = s->tuned_rate[0] * 1e3;
+    trial_rates[1] = s->tuned_rate[1] * 1e3;
+  }
   return BNNHMC_OK;
 }
 

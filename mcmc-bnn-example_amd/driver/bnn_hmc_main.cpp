@@ -260,6 +260,14 @@ int main(int argc, char** argv) {
               "evaluations, %.1f evals/s (device %.0fms).\n",
               hmc.burn_in, hmc.n_samples, hmc.leapfrog_steps, t_ms, evals, evals / (t_ms * 1e-3),
               kernel_ms);
+  int per_launch = 0, per_chain = 0;
+  double trial[2] = {0.0, 0.0};
+  CHECK(bnnhmc_get_batching(s, &per_launch, &per_chain, trial));
+  std::printf("Launches of %d chain(s) on %d workgroups each", per_launch, per_chain);
+  if (trial[0] > 0.0)
+    std::printf(" (last timed pair: rows of a launch within the memory-side cache %.0f evals/s, as many chains "
+                "as fit the device %.0f evals/s)", trial[0], trial[1]);
+  std::printf(".\n");
   if (o.windows * o.chains == 1)
     std::printf("Expected time for 200 sequential passes: %.3fh. Good bye!\n", 200 * (t_ms / 3600000.0));
   CHECK(bnnhmc_destroy(s));

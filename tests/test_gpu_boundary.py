@@ -253,40 +253,60 @@ def test_step_operator_failure_record_survives_later_steps(pkg, lib, orc, monkey
 
 
 # ------------------------------------------------------------------------------------------------
-# automatic batches keep the rows of their windows inside the memory-side cache
+# automatic batches: the rows of a launch inside the memory-side cache, or as many chains as fit the device
 # ------------------------------------------------------------------------------------------------
-def test_automatic_batches_are_cut_to_the_memory_side_cache(pkg, lib, orc, monkeypatch):
-    """With the automatic group size a launch takes no more windows than 192 MB of rows: 32 windows of
-    58368 x 22 (172 MB) on 8 workgroups each where 64 would fit the device on 4; chains that share a window
-    share its rows (32 windows x 2 chains: 64 on 4); small windows are not cut.  The cut only changes how
-    the chains are laid over the device: the same transitions with the limit lifted (the measurement switch
-    BNNHMC_RESIDENT_MB=0) take the same decisions and differ by the rounding of a different group size."""
+def test_automatic_batches_have_two_shapes_and_the_faster_is_measured(pkg, lib, orc, monkeypatch):
+    """With the automatic group size a sampler starts with launches whose windows' rows stay within 192 MB:
+    32 windows of 58368 x 22 (172 MB) on 8 workgroups each where 64 would fit the device on 4; chains that
+    share a window share its rows (32 windows x 2 chains: 64 on 4); small windows are not cut.  A call long
+    enough to hold a launch of each shape times both and goes on with the faster.  Whichever runs, only the
+    layout over the device changes: the same transitions with the limit lifted (the measurement switch
+    BNNHMC_RESIDENT_MB=0) or with the timing switched off (BNNHMC_BATCH_TUNE=0) take the same decisions and
+    differ by the rounding of a different group size."""
     n_full = 58368
-    hmc = lib.default_hmc(leapfrog_steps=3, burn_in=0, n_samples=2, eps0=2e-5, seed=9)
-    model = lib.default_model(n=n_full, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
+    # (a smooth posterior: with the benchmark's sigma = 0.01 log alpha is a difference of sums of order 1e8
+    # and moves by 0.1 with the rounding of another group size)
+    hmc = lib.default_hmc(leapfrog_steps=3, burn_in=0, n_samples=10, eps0=0.005, seed=9)
+    model = lib.default_model(n=n_full, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=2.0, prior_scale=0.05)
 
-    def run(n_windows, cpw, m=model):
-        s = lib.create(m, hmc, lib.default_launch(), n_windows, cpw)
-        b = s.batching()
+    def run(n_windows, cpw, n_trans):
+        s = lib.create(model, hmc, lib.default_launch(), n_windows, cpw)
+        before = s.batching()
         for w in range(n_windows):
             s.generate_window(w, teacher_scale=0.1, noise_sigma=0.01)
         s.init_chains(None)
-        s.run(2)
-        out = [s.get_samples(c) for c in (0, n_windows * cpw - 1)], [s.get_traces(c) for c in (0, n_windows * cpw - 1)]
+        s.run(n_trans)
+        last = n_windows * cpw - 1
+        out = dict(before=before, after=s.batching(), rates=s.batch_trial_rates(),
+                   samples=[s.get_samples(c) for c in (0, last)], traces=[s.get_traces(c) for c in (0, last)])
         s.close()
-        return b, out
+        return out
 
-    say("64 windows of 58368 rows, automatic group size")
-    b_cut, (smp_cut, tr_cut) = run(64, 1)
-    assert b_cut == (32, 8), b_cut
+    def same_chains(a, b):
+        for x, y, tx, ty in zip(a["samples"], b["samples"], a["traces"], b["traces"]):
+            assert np.array_equal(tx["accept"], ty["accept"])
+            assert np.allclose(tx["log_acpt"], ty["log_acpt"], rtol=2e-3, atol=1e-2), (tx["log_acpt"], ty["log_acpt"])
+            assert x.shape == y.shape and np.max(np.abs(x - y)) <= 1e-5 * np.max(np.abs(y))
+
+    say("64 windows of 58368 rows, automatic group size, 10 transitions: both shapes are timed")
+    tuned = run(64, 1, 10)               # 128 quanta of 5 transitions: one launch of 32, one of 64, then the faster
+    assert tuned["before"] == (32, 8), tuned["before"]
+    assert tuned["after"] in ((32, 8), (64, 4)), tuned["after"]
+    assert tuned["rates"][0] > 0 and tuned["rates"][1] > 0
+    say("  trial: %.0f evals/s cache-resident, %.0f evals/s device-wide -> %d x %d" % (tuned["rates"] + tuned["after"]))
+    assert (tuned["after"] == (64, 4)) == (tuned["rates"][1] > tuned["rates"][0])
+    short = run(64, 1, 2)                # no quantum of 5 transitions: nothing is timed
+    assert short["after"] == (32, 8) and short["rates"] == (0.0, 0.0)
+    monkeypatch.setenv("BNNHMC_BATCH_TUNE", "0")
+    fixed = run(64, 1, 10)
+    assert fixed["after"] == (32, 8) and fixed["rates"] == (0.0, 0.0)
+    monkeypatch.delenv("BNNHMC_BATCH_TUNE")
     monkeypatch.setenv("BNNHMC_RESIDENT_MB", "0")
-    b_all, (smp_all, tr_all) = run(64, 1)
-    assert b_all == (64, 4), b_all
+    wide = run(64, 1, 10)
+    assert wide["before"] == wide["after"] == (64, 4) and wide["rates"] == (0.0, 0.0)
     monkeypatch.delenv("BNNHMC_RESIDENT_MB")
-    for a, b, ta, tb in zip(smp_cut, smp_all, tr_cut, tr_all):
-        assert np.array_equal(ta["accept"], tb["accept"])
-        assert np.allclose(ta["log_acpt"], tb["log_acpt"], rtol=2e-3, atol=1e-2), (ta["log_acpt"], tb["log_acpt"])
-        assert np.max(np.abs(a - b)) <= 1e-5 * np.max(np.abs(b))
+    same_chains(tuned, fixed)
+    same_chains(wide, fixed)
     say("32 windows x 2 chains")
     s = lib.create(model, hmc, lib.default_launch(), 32, 2)
     assert s.batching() == (64, 4), s.batching()
