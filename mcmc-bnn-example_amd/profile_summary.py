@@ -22,6 +22,14 @@ def counter_totals(path, kernel_substr):
     return agg
 
 
+def median_launch(tot, size):
+    """(dispatch, counters) of the launch of median size among the launches of transitions (the evaluation
+    launches, thousands of times smaller, are left out): the shape most of the run was spent in"""
+    items = sorted(tot.items(), key=lambda kv: size(kv[1]))
+    big = [kv for kv in items if size(kv[1]) >= 0.02 * size(items[-1][1])]
+    return big[len(big) // 2]
+
+
 def bench_json(path):
     try:
         return json.loads(open(path).read().strip().splitlines()[-1])
@@ -105,9 +113,9 @@ def main(out):
     sq = find(os.path.join(out, "pmc_SQ"), "*counter_collection.csv")
     if sq:
         tot = counter_totals(sq, "hmc_kernel")
-        disp, v = max(tot.items(), key=lambda kv: kv[1].get("GRBM_GUI_ACTIVE", 0))
+        disp, v = median_launch(tot, lambda c: c.get("GRBM_GUI_ACTIVE", 0))
         simd_cycles = 1024.0 * v["GRBM_GUI_ACTIVE"] / 8.0  # 8 XCDs report, 1024 SIMDs
-        lines.append("SQ counters, hmc_kernel dispatch %s (fractions of all SIMD cycles):" % disp)
+        lines.append("SQ counters, hmc_kernel dispatch %s, the median launch of transitions (fractions of all SIMD cycles):" % disp)
         lines.append("  MFMA pipe busy %.3f | VALU (non-MFMA) active %.3f | any instruction active %.3f | "
                      "VALU insts per MFMA %.2f" % (
                          v["SQ_VALU_MFMA_BUSY_CYCLES"] / simd_cycles, 4 * v["SQ_ACTIVE_INST_VALU"] / simd_cycles,
@@ -116,9 +124,9 @@ def main(out):
     tcc = find(os.path.join(out, "pmc_TCC"), "*counter_collection.csv")
     if tcc:
         tot = counter_totals(tcc, "hmc_kernel")
-        disp, v = max(tot.items(), key=lambda kv: kv[1].get("TCC_HIT_sum", 0) + kv[1].get("TCC_MISS_sum", 0))
+        disp, v = median_launch(tot, lambda c: c.get("TCC_HIT_sum", 0) + c.get("TCC_MISS_sum", 0))
         hit, miss = v["TCC_HIT_sum"], v["TCC_MISS_sum"]
-        lines.append("L2 (TCC), hmc_kernel dispatch %s: hits %.4g, misses %.4g -> hit rate %.3f; read requests to "
+        lines.append("L2 (TCC), hmc_kernel dispatch %s, the median launch of transitions: hits %.4g, misses %.4g -> hit rate %.3f; read requests to "
                      "the fabric %.4g of which marked DRAM %.4g" % (disp, hit, miss, hit / max(1.0, hit + miss),
                                                                    v["TCC_EA0_RDREQ_sum"], v["TCC_EA0_RDREQ_DRAM_sum"]))
     text = "\n".join(lines)
