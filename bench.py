@@ -265,7 +265,7 @@ def main():
             "batch_shape_trial": None if trial[0] <= 0 else (
                 "the library timed one launch of each shape at the start of the %s: rows of a launch within the "
                 "memory-side cache %.0f evals/s, as many chains as fit the device %.0f evals/s" % (
-                    "job" if args.full else "warm-up call", trial[0], trial[1])),
+                    "last call of the job" if args.full else "warm-up call", trial[0], trial[1])),
             "workgroups_last_launch": tm1["workgroups"], "compute_units": cus,
             "transitions_per_launch": args.transitions_per_launch,
             "eps0": float(hmc.eps0), "adapt_steps": int(hmc.adapt_steps),
