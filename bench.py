@@ -7,9 +7,10 @@ N(0, 0.01^2) noise, Gaussian likelihood, Gaussian weight prior), one chain per w
 leapfrog steps per transition, all 200 windows resident in HBM (1.07 GB).  A "step" is one HMC transition
 (momentum resampling, 1000 fused leapfrog gradient evaluations, log accept ratio, Metropolis decision,
 sample store) of every one of the 200 windows: the chains take turns, five transitions at a time, on
-launches of 32 chains at 8 workgroups per chain (the rows of 32 windows, 172 MB, stay in the memory-side
-cache from one leapfrog step to the next); what does not fill such a launch runs as 16 chains at 16, 8 at
-32, ... workgroups per chain, always over all 256 compute units.  The warm-up transitions
+launches of 64 chains at 4 workgroups per chain (of the rows of 64 windows, 344 MB, the 256 MB memory-side
+cache serves most from one leapfrog step to the next, because a wave walks its tiles back and forth) or of 128
+chains at 2, whichever the library measures to be faster in the warm-up call; what does not fill such a launch
+runs as 32 chains at 8, 16 at 16, ... workgroups per chain, always over all 256 compute units.  The warm-up transitions
 are the burn-in (nothing stored), the timed ones store their samples.  The metric is leapfrog gradient
 evaluations per second; the minutes for 200 windows x (100 burn-in + 800 samples) are 900 steps plus the
 bootstrap evaluation, and --full runs that whole job.
@@ -50,7 +51,7 @@ def batch_plan(n_chains, resident_wgs, cus_per_chain, wide, max_chains):
     """[(chains, workgroups per chain)] of the launches that cover n_chains, as the library lays them out:
     a fixed group size when one is configured (the 64->128->1 default is 4), otherwise the largest
     power-of-two number of chains that is left and fits (max_chains: what the library says fits, which
-    also keeps a launch's rows inside the memory-side cache), spread over the whole device; a batch that
+    may keep a launch's rows within 1.4 times the memory-side cache), spread over the whole device; a batch that
     leaves compute units idle gets its groups doubled while they still fit."""
     def widen(g, b):
         while g * 2 * b <= resident_wgs and g * 2 <= 256:
@@ -263,8 +264,8 @@ def main():
                 if not wide and not launch.cus_per_chain and len(plan) > 1
                 else ", ".join("%d x %d" % bg for bg in plan)),
             "batch_shape_trial": None if trial[0] <= 0 else (
-                "the library timed one launch of each shape at the start of the %s: rows of a launch within the "
-                "memory-side cache %.0f evals/s, as many chains as fit the device %.0f evals/s" % (
+                "the library timed one launch of each shape at the start of the %s: rows of a launch within 1.4 "
+                "times the memory-side cache %.0f evals/s, as many chains as fit the device %.0f evals/s" % (
                     "last call of the job" if args.full else "warm-up call", trial[0], trial[1])),
             "workgroups_last_launch": tm1["workgroups"], "compute_units": cus,
             "transitions_per_launch": args.transitions_per_launch,

@@ -75,8 +75,8 @@ typedef struct bnnhmc_launch {
                       /* 22 -> 40 -> 1: a batch is the largest power-of-two number of chains that */
                       /* fits, spread over the whole device (one chain: 256 workgroups; 128 or     */
                       /* more chains on 256 CUs: 2 each) -- or, where that is measured to be       */
-                      /* faster, the largest whose windows' rows stay within 192 MB, the           */
-                      /* memory-side cache (32 windows of 58368 x 22: 8 each; see                  */
+                      /* faster, the largest whose windows' rows stay within 358 MB, most of       */
+                      /* which the memory-side cache serves (64 windows of 58368 x 22: 4 each; see */
                       /* bnnhmc_get_batching); more chains than fit take turns on such             */
                       /* batches, transitions_per_launch transitions at a time, and what does not  */
                       /* fill a batch runs in smaller, wider ones.  64 -> 128 -> 1: 4, a smaller    */
@@ -271,16 +271,16 @@ int bnnhmc_final_loss(bnnhmc_sampler* s, int chain, double* loss1, double* loss2
 /* How bnnhmc_run lays the sampler's chains over the device at present: chains in a full launch and
  * workgroups per chain in it.  With the automatic group size (cus_per_chain = 0) of the 22 -> 40 -> 1 kernel
  * a launch takes the largest power-of-two number of chains that fits the device at one workgroup per chain;
- * where the rows of so many windows exceed 192 MB there is a second shape, the largest such number whose
- * windows' rows stay within 192 MB, so that after the first leapfrog step they are served by the
- * memory-side cache instead of HBM (200 windows of 58368 x 22: 32 at a time on 8 workgroups each, against
- * 128 on 2).  Which is faster depends on the card and on the data (the card is power-limited: HBM traffic
- * costs shader clock when the arithmetic is dense).  A sampler starts with the cache-resident shape; a
- * bnnhmc_run call that is long enough (a launch of each shape fits in it) first runs one launch of each,
- * timed, and goes on with the faster, and so do later calls, which time the two again after every 2000
- * launches' worth of chains.  trial_rates (may be NULL) receives the gradient evaluations per second of the
- * last such pair, cache-resident shape first; zeros if none was run.  No counterpart in the reference (one
- * chain per process). */
+ * where the rows of so many windows exceed 358 MB (1.4 times the memory-side cache, which serves most of a
+ * batch of that size because a wave walks its tiles back and forth) there is a second shape, the largest
+ * such number whose windows' rows stay within 358 MB (200 windows of 58368 x 22: 64 at a time on 4
+ * workgroups each, against 128 on 2).  Which is faster depends on the card and on the data (the card is
+ * power-limited: HBM traffic costs shader clock when the arithmetic is dense).  A sampler starts with the
+ * shape within the budget; a bnnhmc_run call that is long enough (a launch of each shape fits in it) first
+ * runs one launch of each, timed, and goes on with the faster, and so do later calls, which time the two
+ * again after every 2000 launches' worth of chains.  trial_rates (may be NULL) receives the gradient
+ * evaluations per second of the last such pair, the shape within the budget first; zeros if none was run.
+ * No counterpart in the reference (one chain per process). */
 int bnnhmc_get_batching(bnnhmc_sampler* s, int* chains_per_launch, int* workgroups_per_chain,
                         double* trial_rates);
 

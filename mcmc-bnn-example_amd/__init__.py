@@ -326,7 +326,7 @@ class Sampler:
         return b.value, g.value
 
     def batch_trial_rates(self):
-        """gradient evaluations/s of the last timed pair of launches: (cache-resident shape, device-wide shape)"""
+        """gradient evaluations/s of the last timed pair of launches: (the shape within the row budget, the device-wide shape)"""
         r = (C.c_double * 2)()
         self.lib.check(self.lib.c.bnnhmc_get_batching(self.h, None, None, r))
         return r[0], r[1]

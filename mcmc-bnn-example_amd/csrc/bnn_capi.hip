@@ -129,22 +129,25 @@ int env_pipeline() {
   const char* e = getenv("BNNHMC_PIPELINE");
   return e && *e ? atoi(e) : 0;
 }
-// The rows of the windows of a launch are read again at every leapfrog step.  A batch whose windows fit the
-// 256 MB memory-side cache gets them from there after the first step; a wider one streams them from HBM
-// (2.3 TB/s at 128 windows of 58368 x 22 on 2 workgroups each).  What that costs depends on the card --
-// evaluations/s of 128 windows at 2 workgroups per chain / 64 at 4 / 32 at 8, each batch filling the device:
-// 419 k / 415 k / 415 k on one MI355X, 395 k / 396 k / 415 k on another, and with the reference's Student-t
-// model, whose saturated hidden units put zeros into the second contraction, 427 k / - / 406 k.  The card is
-// power-limited: with the dense Gaussian workload the HBM traffic of the wide batch lowers the shader clock from
-// 2.36 to 2.23 GHz, with the lighter one it does not and the narrow groups' smaller share of exchange time wins.
+// The rows of the windows of a launch are read again at every leapfrog step, and a wave walks its tiles forwards
+// in one step and backwards in the next (MfmaHybridLayer), so a step starts with the rows the step before ended
+// on: of a batch whose rows are D bytes the 256 MB memory-side cache serves about 256 MB / D, the rest comes from
+// HBM (2.3 TB/s at 128 windows of 58368 x 22).  What that traffic costs depends on the card and on the data.  The
+// card is power-limited: with the dense operands of the Gaussian benchmark 128 windows at 2 workgroups per chain
+// streamed from HBM run at a shader clock of 2.23 GHz on some cards where a cache-resident batch runs at 2.36
+// (same cycles per tile), on others they do not lose clock; the reference's Student-t model, whose saturated hidden
+// units put zeros into the second contraction, has power to spare everywhere, and then the narrow groups' smaller
+// share of exchange time wins.  Evaluations/s of 128 windows at 2 workgroups per chain / 64 at 4 / 32 at 8, every
+// CU busy, one card: Gaussian 420 k / 423 k / 413 k, Student-t 428 k / 420 k / 406 k (walking forwards only, the
+// Gaussian figures were 416 k / 411 k / 414 k there and 395 k / 396 k / 415 k on a card that loses clock).
 // So with the automatic group size a sampler whose chains take turns has two batch shapes -- the largest that
-// fits the device, and the largest whose windows fit this budget (32 of that size: 172 MB) -- and bnnhmc_run
-// times one launch of each at the start of a call and goes on with the faster (tune_batch below).
+// fits the device, and the largest whose windows' rows fit this budget, 1.4 times the cache (64 windows of that
+// size: 344 MB) -- and bnnhmc_run times one launch of each at the start of a call and goes on with the faster.
 // BNNHMC_RESIDENT_MB=<n> replaces the budget for measurements (0: no limit, one shape);
-// BNNHMC_BATCH_TUNE=0 switches the timing off (the cache-resident shape is then used throughout).
+// BNNHMC_BATCH_TUNE=0 switches the timing off (the shape within the budget is then used throughout).
 size_t resident_row_budget() {
   const char* e = getenv("BNNHMC_RESIDENT_MB");
-  const long mb = e && *e ? atol(e) : 192;
+  const long mb = e && *e ? atol(e) : 358;
   return mb <= 0 ? (size_t)0 : (size_t)mb << 20;
 }
 // chains of a batch whose windows' rows fit the budget (0: no limit)
@@ -563,9 +566,9 @@ struct bnnhmc_sampler {
   hipStream_t stream = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   hipEvent_t ev_t0 = nullptr, ev_t1 = nullptr;  // around one launch while the batch shape is being chosen
-  int batch_cap = 0;        // chains of a batch whose windows' rows fit the memory-side cache (0: no such limit)
+  int batch_cap = 0;        // chains of a batch whose windows' rows fit resident_row_budget() (0: no such limit)
   int batch_limit = 0;      // the limit bnnhmc_run applies at present: batch_cap or 0 (what fits the device)
-  double tuned_rate[2] = {0.0, 0.0};  // evaluations per ms of the last trial launches: cache-resident, device-wide
+  double tuned_rate[2] = {0.0, 0.0};  // evaluations per ms of the last trial launches: within the budget, device-wide
   long quanta_since_tune = -1;        // quanta dealt since the shapes were last timed (-1: never)
   // device memory
   float* X = nullptr;

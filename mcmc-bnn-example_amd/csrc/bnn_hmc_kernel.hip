@@ -330,6 +330,8 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
   }
 
   Layer layer;
+  cx.back = leapfrog_walks_back(0, a.L);
+  cx.back_next = cx.back;
   layer.prime(cx);  // the first tiles of the first gradient evaluation
   bool ok = true;
   // optional per-phase cycle accounting (thread 0 of each workgroup)
@@ -397,6 +399,8 @@ __global__ __launch_bounds__(T) void hmc_kernel(const KArgs a) {
       layer.zero_acc();
       BNN_PHASE(1)  // operand fetch from LDS
       const bool last = s == a.L - 1;
+      cx.back = leapfrog_walks_back(s, a.L);
+      cx.back_next = leapfrog_walks_back(last ? 0 : s + 1, a.L);
       if (last) {
         cx.ell_prev = ell_cur;
         cx.ell_new = ell_prop;

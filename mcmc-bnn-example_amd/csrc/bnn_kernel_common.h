@@ -264,7 +264,14 @@ struct StepCtx {
   int* progress;          // LDS, one word per wave: tiles done in this step (null = no balancing)
   int wave, partner;      // this wave and the wave it shares a SIMD with
   float* tile_lds;        // LDS, this wave's copy of the tile it is working on (layers that keep one)
+  int back, back_next;    // this gradient evaluation / the next one walks a wave's tiles backwards (layers that
+                          // alternate; see leapfrog_walks_back)
 };
+
+// Direction of the gradient evaluation of leapfrog step s of L: alternating, and forwards in the last step, so
+// that the gradient a chain keeps is always summed in the same order (a chain restored from a saved position
+// recomputes it with a one-step launch and must get the same bits).
+__device__ __forceinline__ int leapfrog_walks_back(int s, int L) { return (L - 1 - s) & 1; }
 
 // ------------------------------------------------------------------------------------------------
 // group barrier: all G workgroups of a chain group have published their partials of this step.

@@ -379,16 +379,25 @@ struct MfmaHybridLayer {
     return fast_end;
   }
 
+  // A wave walks its run of tiles forwards in one gradient evaluation and backwards in the next (cx.back,
+  // cx.back_next): what it read last -- what the caches most likely still hold when the rows of all chains in
+  // flight exceed them -- is what it reads first.  The partial sums of a backward evaluation are added in the
+  // opposite order, so the direction is a function of the leapfrog step alone, and the last step of a trajectory,
+  // whose gradient a chain carries into its next transition (and a resumed chain computes afresh), always goes
+  // forwards.
   TileRaw pa, pb;  // the first two tiles of the next evaluation (see MfmaLayer)
+  // tile number k of an evaluation's walk over [tb, te)
+  static __device__ __forceinline__ int walk(int tb, int te, int k, int back) { return back ? te - 1 - k : tb + k; }
   __device__ __forceinline__ void prime(const StepCtx& cx) {
     const int tb = cx.tile_begin, te = fast_end_of(cx);
     if (te <= tb) return;
     const int lane = opaque_tid() & 63;
     const LoadPlan lp = load_plan(lane & 15, lane >> 4);
+    const int back = __builtin_amdgcn_readfirstlane(cx.back);
     preset(pa);
     preset(pb);
-    issue_tile(pa, cx, lp, tb);
-    issue_tile(pb, cx, lp, tb + 1 < te ? tb + 1 : tb);
+    issue_tile(pa, cx, lp, __builtin_amdgcn_readfirstlane(walk(tb, te, 0, back)));
+    issue_tile(pb, cx, lp, __builtin_amdgcn_readfirstlane(walk(tb, te, tb + 1 < te ? 1 : 0, back)));
     wait_tile<0>(pa);
     wait_tile<0>(pb);
   }
@@ -398,15 +407,27 @@ struct MfmaHybridLayer {
                                                 int q) {
     const LoadPlan lp = load_plan(n, q);
     float* tile = cx.tile_lds;
-    int nxt = te - tb > 2 ? tb + 2 : tb;
+    // the loads run two tiles ahead of the arithmetic along the walk, into the next evaluation's (which goes
+    // the other way) at the end of this one's
+    const int back = __builtin_amdgcn_readfirstlane(cx.back);
+    const int back_next = __builtin_amdgcn_readfirstlane(cx.back_next);
+    const int len = te - tb;
+    int nk = 2, nback = back;
+    while (nk >= len) {  // (a run of one tile is the same tile in either direction)
+      nk -= len;
+      nback = back_next;
+    }
     auto issue = [&](TileRaw& r) {
-      issue_tile(r, cx, lp, nxt);
-      nxt = nxt + 1 == te ? tb : nxt + 1;
+      issue_tile(r, cx, lp, __builtin_amdgcn_readfirstlane(walk(tb, te, nk, nback)));
+      if (++nk == len) {
+        nk = 0;
+        nback = back_next;
+      }
     };
-    auto compute = [&](TileRaw& r, int t) {
+    auto compute = [&](TileRaw& r, int i) {  // i: tb + position in the walk
       r.t.xa[0] = f2{r.xa01[0], r.xa01[1]};
       r.t.xa[1] = f2{r.xa01[2], r.xa01[3]};
-      compute_tile<LIK, LAST, true>(r.t, tile, cx, mc, t * 16, n, q);
+      compute_tile<LIK, LAST, true>(r.t, tile, cx, mc, walk(tb, te, i - tb, back) * 16, n, q);
     };
     TileRaw& A = pa;
     TileRaw& B = pb;

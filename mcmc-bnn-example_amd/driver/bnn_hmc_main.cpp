@@ -265,7 +265,7 @@ int main(int argc, char** argv) {
   CHECK(bnnhmc_get_batching(s, &per_launch, &per_chain, trial));
   std::printf("Launches of %d chain(s) on %d workgroups each", per_launch, per_chain);
   if (trial[0] > 0.0)
-    std::printf(" (last timed pair: rows of a launch within the memory-side cache %.0f evals/s, as many chains "
+    std::printf(" (last timed pair: rows of a launch within 1.4 times the memory-side cache %.0f evals/s, as many chains "
                 "as fit the device %.0f evals/s)", trial[0], trial[1]);
   std::printf(".\n");
   if (o.windows * o.chains == 1)

@@ -253,12 +253,12 @@ def test_step_operator_failure_record_survives_later_steps(pkg, lib, orc, monkey
 
 
 # ------------------------------------------------------------------------------------------------
-# automatic batches: the rows of a launch inside the memory-side cache, or as many chains as fit the device
+# automatic batches: the rows of a launch within 1.4 times the memory-side cache, or as many chains as fit
 # ------------------------------------------------------------------------------------------------
 def test_automatic_batches_have_two_shapes_and_the_faster_is_measured(pkg, lib, orc, monkeypatch):
-    """With the automatic group size a sampler starts with launches whose windows' rows stay within 192 MB:
-    32 windows of 58368 x 22 (172 MB) on 8 workgroups each where 64 would fit the device on 4; chains that
-    share a window share its rows (32 windows x 2 chains: 64 on 4); small windows are not cut.  A call long
+    """With the automatic group size a sampler starts with launches whose windows' rows stay within 358 MB:
+    64 windows of 58368 x 22 (344 MB) on 4 workgroups each where 128 would fit the device on 2; chains that
+    share a window share its rows (64 windows x 2 chains: 128 on 2); small windows are not cut.  A call long
     enough to hold a launch of each shape times both and goes on with the faster.  Whichever runs, only the
     layout over the device changes: the same transitions with the limit lifted (the measurement switch
     BNNHMC_RESIDENT_MB=0) or with the timing switched off (BNNHMC_BATCH_TUNE=0) take the same decisions and
@@ -288,28 +288,29 @@ def test_automatic_batches_have_two_shapes_and_the_faster_is_measured(pkg, lib, 
             assert np.allclose(tx["log_acpt"], ty["log_acpt"], rtol=2e-3, atol=1e-2), (tx["log_acpt"], ty["log_acpt"])
             assert x.shape == y.shape and np.max(np.abs(x - y)) <= 1e-5 * np.max(np.abs(y))
 
-    say("64 windows of 58368 rows, automatic group size, 10 transitions: both shapes are timed")
-    tuned = run(64, 1, 10)               # 128 quanta of 5 transitions: one launch of 32, one of 64, then the faster
-    assert tuned["before"] == (32, 8), tuned["before"]
-    assert tuned["after"] in ((32, 8), (64, 4)), tuned["after"]
+    say("128 windows of 58368 rows, automatic group size, 10 transitions: both shapes are timed")
+    tuned = run(128, 1, 10)              # 256 quanta of 5 transitions: one launch of 64, one of 128, then the faster
+    assert tuned["before"] == (64, 4), tuned["before"]
+    assert tuned["after"] in ((64, 4), (128, 2)), tuned["after"]
     assert tuned["rates"][0] > 0 and tuned["rates"][1] > 0
-    say("  trial: %.0f evals/s cache-resident, %.0f evals/s device-wide -> %d x %d" % (tuned["rates"] + tuned["after"]))
-    assert (tuned["after"] == (64, 4)) == (tuned["rates"][1] > tuned["rates"][0])
-    short = run(64, 1, 2)                # no quantum of 5 transitions: nothing is timed
-    assert short["after"] == (32, 8) and short["rates"] == (0.0, 0.0)
+    say("  trial: %.0f evals/s within the row budget, %.0f evals/s device-wide -> %d x %d" % (
+        tuned["rates"] + tuned["after"]))
+    assert (tuned["after"] == (128, 2)) == (tuned["rates"][1] > tuned["rates"][0])
+    short = run(128, 1, 2)               # no quantum of 5 transitions: nothing is timed
+    assert short["after"] == (64, 4) and short["rates"] == (0.0, 0.0)
     monkeypatch.setenv("BNNHMC_BATCH_TUNE", "0")
-    fixed = run(64, 1, 10)
-    assert fixed["after"] == (32, 8) and fixed["rates"] == (0.0, 0.0)
+    fixed = run(128, 1, 10)
+    assert fixed["after"] == (64, 4) and fixed["rates"] == (0.0, 0.0)
     monkeypatch.delenv("BNNHMC_BATCH_TUNE")
     monkeypatch.setenv("BNNHMC_RESIDENT_MB", "0")
-    wide = run(64, 1, 10)
-    assert wide["before"] == wide["after"] == (64, 4) and wide["rates"] == (0.0, 0.0)
+    wide = run(128, 1, 10)
+    assert wide["before"] == wide["after"] == (128, 2) and wide["rates"] == (0.0, 0.0)
     monkeypatch.delenv("BNNHMC_RESIDENT_MB")
     same_chains(tuned, fixed)
     same_chains(wide, fixed)
-    say("32 windows x 2 chains")
-    s = lib.create(model, hmc, lib.default_launch(), 32, 2)
-    assert s.batching() == (64, 4), s.batching()
+    say("64 windows x 2 chains")
+    s = lib.create(model, hmc, lib.default_launch(), 64, 2)
+    assert s.batching() == (128, 2), s.batching()
     s.close()
     small = lib.default_model(n=4096, lik_kind=pkg.LIK_GAUSSIAN, lik_scale=0.01, prior_scale=0.1)
     s = lib.create(small, hmc, lib.default_launch(), 200, 1)

@@ -85,7 +85,7 @@ def test_burn_in_transitions_50_to_100_at_full_size(config0_chain, orc):
     c = config0_chain
     tr, starts = c["traces"], c["starts"]
     log_target = float(np.log(np.float32(0.2)))
-    n_acc = n_rej_finite = n_div = n_unclear = n_eps_checked = n_big = 0
+    n_acc = n_rej_finite = n_div = n_unclear = n_eps_checked = n_big = n_chaotic = 0
     t0 = time.time()
     for t in range(50, 100):
         w, eps = starts[t]
@@ -95,8 +95,24 @@ def test_burn_in_transitions_50_to_100_at_full_size(config0_chain, orc):
         # (an unstable trajectory amplifies every rounding difference: only its verdict is compared; the
         # uniform is never below log FLT_MIN = -87.3)
         divergent = (not np.isfinite(la_ref)) or la_ref < -1e3
+
+        def at_the_stability_limit():
+            # the oracle's own ratio from a start one ulp away: where that moves it by more than half (or
+            # changes its sign), the trajectory sits on the integrator's stability limit and amplifies any
+            # rounding difference without bound -- there is no verdict to compare
+            # (while the chain still sits at the all-zero start there is no ulp to add to the position: the step
+            # size is moved by one instead)
+            w_up = np.nextafter(w, np.float32(np.inf)).astype(np.float32)
+            eps_up = eps if np.any(w != 0) else np.nextafter(np.float32(eps), np.float32(1))
+            la_up = float(orc.run_chain_from(c["om"], c["oh"], c["X"], c["y"], w_up, float(eps_up), t, 1)["log_acpt"][0])
+            say("  t=%d eps %.3e log alpha gpu %.6g oracle %.6g, oracle one ulp away %.6g" % (t, eps, la_gpu, la_ref, la_up))
+            return (not np.isfinite(la_up)) or (not np.isfinite(la_ref)) or abs(la_up - la_ref) > 0.5 * abs(la_ref)
+
+        if divergent and not ((not np.isfinite(la_gpu)) or la_gpu < -1e2):
+            assert abs(la_gpu) > 1e2 and at_the_stability_limit(), (t, la_gpu, la_ref)
+            n_chaotic += 1
+            continue
         if divergent:
-            assert (not np.isfinite(la_gpu)) or la_gpu < -1e2, (t, la_gpu, la_ref)
             assert tr["accept"][t] == 0 and ref["accept"][0] == 0
             assert np.float32(tr["eps"][t]).tobytes() == np.float32(ref["eps"][0]).tobytes(), t
             n_div += 1
@@ -106,7 +122,11 @@ def test_burn_in_transitions_50_to_100_at_full_size(config0_chain, orc):
             # integrator: ratios of 1e2 .. 1e6 that differ by tens of percent between implementations (and
             # between two oracle runs one ulp apart); accepted whatever the uniform, step size incremented
             say("  t=%d eps %.3e log alpha gpu %.6g oracle %.6g: accept whatever the uniform" % (t, eps, la_gpu, la_ref))
-            assert la_gpu > 10.0 and tr["accept"][t] == 1 and ref["accept"][0] == 1, (t, la_gpu, la_ref)
+            if not (la_gpu > 10.0):
+                assert ((not np.isfinite(la_gpu)) or abs(la_gpu) > 1e2) and at_the_stability_limit(), (t, la_gpu, la_ref)
+                n_chaotic += 1
+                continue
+            assert tr["accept"][t] == 1 and ref["accept"][0] == 1, (t, la_gpu, la_ref)
             assert np.float32(tr["eps"][t]).tobytes() == np.float32(ref["eps"][0]).tobytes(), t
             n_acc += 1
             n_big += 1
@@ -134,13 +154,14 @@ def test_burn_in_transitions_50_to_100_at_full_size(config0_chain, orc):
         else:
             n_rej_finite += 1
     say("transitions 50..99: %d divergent rejects, %d accepts (%d of them at ratios above 100), %d rejects at a "
-        "finite ratio, %d inside the margin, %d step sizes compared bit for bit; oracle time %.0f s" % (
-            n_div, n_acc, n_big, n_rej_finite, n_unclear, n_eps_checked + n_div + n_big, time.time() - t0))
+        "finite ratio, %d inside the margin, %d at the stability limit (no verdict), %d step sizes compared bit "
+        "for bit; oracle time %.0f s" % (
+            n_div, n_acc, n_big, n_rej_finite, n_unclear, n_chaotic, n_eps_checked + n_div + n_big, time.time() - t0))
     # what this stretch of the chain holds (eps0 = 0.01 needs about 65 decrements before a trajectory is
     # stable, so the first 90 transitions hold fewer than 15 rejects at a finite ratio; the adapted leg below
     # adds 20 transitions of which about two thirds reject)
     assert n_div >= 10 and n_acc >= 20 and n_acc - n_big >= 8 and n_rej_finite >= 4
-    assert n_unclear <= 8
+    assert n_unclear <= 8 and n_chaotic <= 3
 
 
 def _log_alpha_f64(orc, X, y, w0, eps, t):
@@ -359,8 +380,9 @@ def test_1600_samples_at_reduced_size(pkg, lib, orc):
 
 
 # ------------------------------------------------------------------------------------------------
-# configs[2] batching: 200 windows of 58368 rows as six batches of 32 (8 workgroups per chain: the rows of a
-# batch stay in the memory-side cache) and a last batch of 8 (widened to 32 workgroups per chain)
+# configs[2] batching: 200 windows of 58368 rows as three batches of 64 (4 workgroups per chain: the shape a
+# sampler starts with, its rows within 1.4 times the memory-side cache) and a last batch of 8 (widened to 32
+# workgroups per chain)
 # ------------------------------------------------------------------------------------------------
 def test_200_windows_are_batched_without_crosstalk(pkg, lib, orc):
     # a step size small enough that trajectories from the all-zero start are accepted
@@ -377,18 +399,17 @@ def test_200_windows_are_batched_without_crosstalk(pkg, lib, orc):
     big.run(burn + keep)
     assert big.timing()["grad_evals"] == 200 * 2 * L
     checks = {}
-    for chain in (0, 31, 32, 63, 64, 150, 191, 192, 199):
+    for chain in (0, 63, 64, 127, 128, 150, 191, 192, 199):
         checks[chain] = (big.get_samples(chain), big.get_traces(chain), big.get_chain_state(chain),
                          big.get_window_data(chain) if chain in (0, 150, 199) else None)
         assert np.all(np.isfinite(checks[chain][0])) and checks[chain][2]["transitions_done"] == 2
         assert checks[chain][2]["n_accepted"] >= 1 and np.abs(checks[chain][0]).max() > 0
     big.close()
-    assert not np.array_equal(checks[31][0], checks[32][0])       # different windows, different chains
-    # the rows of 32 such windows fit the memory-side cache, so the 200 chains ran in six batches of 32 at 8
-    # workgroups per chain and a tail batch of 8 at 32: each chain must equal, bit for bit, a sampler that
-    # holds only that window and is launched that way
-    assert big_batching == (32, 8), big_batching
-    for chain, G in ((0, 8), (150, 8), (199, 32)):
+    assert not np.array_equal(checks[63][0], checks[64][0])       # different windows, different chains
+    # the 200 chains ran in three batches of 64 at 4 workgroups per chain and a tail batch of 8 at 32: each chain
+    # must equal, bit for bit, a sampler that holds only that window and is launched that way
+    assert big_batching == (64, 4), big_batching
+    for chain, G in ((0, 4), (150, 4), (199, 32)):
         X, y = checks[chain][3]
         h1 = lib.default_hmc(leapfrog_steps=L, burn_in=burn, n_samples=keep, eps0=eps0, seed=0,
                              adapt_steps=0, chain_id_base=chain)
