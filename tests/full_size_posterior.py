@@ -149,7 +149,7 @@ def compare(fa, fb, fyard=None):
     print("the same statistic between two chains of ONE sampler: max |z| = %.2f, %.1f %% above 3" % (
         zy.max(), 100 * np.mean(zy > 3)))
     same = first >= 50 and z.max() <= 1.5 * zy.max() and np.mean(z > 3) <= np.mean(zy > 3) + 0.1
-    print("verdict: the two implementations are %s than two chains of one implementation" % (
+    print("result: the two implementations are %s than two chains of one implementation" % (
         "no further apart" if same else "FURTHER APART"))
     return 0 if same else 1
 

@@ -92,14 +92,14 @@ def test_burn_in_transitions_50_to_100_at_full_size(config0_chain, orc):
         ref = orc.run_chain_from(c["om"], c["oh"], c["X"], c["y"], w, float(eps), t, 1)
         la_ref, la_gpu = float(ref["log_acpt"][0]), float(tr["log_acpt"][t])
         lu = orc.log_uniform(0, 0, t)
-        # (an unstable trajectory amplifies every rounding difference: only its verdict is compared; the
+        # (an unstable trajectory amplifies every rounding difference: only its outcome (reject) is compared; the
         # uniform is never below log FLT_MIN = -87.3)
         divergent = (not np.isfinite(la_ref)) or la_ref < -1e3
 
         def at_the_stability_limit():
             # the oracle's own ratio from a start one ulp away: where that moves it by more than half (or
             # changes its sign), the trajectory sits on the integrator's stability limit and amplifies any
-            # rounding difference without bound -- there is no verdict to compare
+            # rounding difference without bound -- there is no outcome to compare
             # (while the chain still sits at the all-zero start there is no ulp to add to the position: the step
             # size is moved by one instead)
             w_up = np.nextafter(w, np.float32(np.inf)).astype(np.float32)
@@ -154,7 +154,7 @@ def test_burn_in_transitions_50_to_100_at_full_size(config0_chain, orc):
         else:
             n_rej_finite += 1
     say("transitions 50..99: %d divergent rejects, %d accepts (%d of them at ratios above 100), %d rejects at a "
-        "finite ratio, %d inside the margin, %d at the stability limit (no verdict), %d step sizes compared bit "
+        "finite ratio, %d inside the margin, %d at the stability limit (nothing to compare), %d step sizes compared bit "
         "for bit; oracle time %.0f s" % (
             n_div, n_acc, n_big, n_rej_finite, n_unclear, n_chaotic, n_eps_checked + n_div + n_big, time.time() - t0))
     # what this stretch of the chain holds (eps0 = 0.01 needs about 65 decrements before a trajectory is
