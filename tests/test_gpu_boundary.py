@@ -282,10 +282,16 @@ def test_automatic_batches_have_two_shapes_and_the_faster_is_measured(pkg, lib, 
         s.close()
         return out
 
-    def same_chains(a, b):
-        for x, y, tx, ty in zip(a["samples"], b["samples"], a["traces"], b["traces"]):
-            assert np.array_equal(tx["accept"], ty["accept"])
+    def same_chains(a, b, n_windows=128):
+        for chain, x, y, tx, ty in zip((0, n_windows - 1), a["samples"], b["samples"], a["traces"], b["traces"]):
+            # the same ratios and decisions, except where the uniform sits on the ratio (then neither the later
+            # ratios nor the samples of that chain can be compared)
+            close = [abs(orc.log_uniform(9, chain, k) - float(tx["log_acpt"][k])) < 0.02 for k in range(len(tx["accept"]))]
+            if any(close):
+                say("  chain %d: a uniform within 0.02 of the ratio, decisions not compared" % chain)
+                continue
             assert np.allclose(tx["log_acpt"], ty["log_acpt"], rtol=2e-3, atol=1e-2), (tx["log_acpt"], ty["log_acpt"])
+            assert np.array_equal(tx["accept"], ty["accept"])
             assert x.shape == y.shape and np.max(np.abs(x - y)) <= 1e-5 * np.max(np.abs(y))
 
     say("128 windows of 58368 rows, automatic group size, 10 transitions: both shapes are timed")
